@@ -118,9 +118,11 @@ class PartSpec:
 class LayerCall:
     """One entry of the run order: which layer runs, and whose cache it uses.  ``cache_of`` names an
     earlier entry of the order (by its index in the order); the call then reads that entry's cache
-    and writes none of its own."""
+    and writes none of its own.  ``adds_embedding``: the embedding's rows (the stream as it was before the first
+    entry) are added to the stream right before this entry runs: a range of layers that runs again starts so."""
     layer: int
     cache_of: int | None = None
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

@@ -1,0 +1,347 @@
+// Causal grouped-query softmax attention over the paged cache with the options that the plain attention kernels do not
+// have: a key size and a value size of their own, an RMS norm over the whole q projection and the whole k projection
+// (or per head, or none), biases on q, k and v, a rotation of the first `rot` dimensions of each head, a sliding
+// window, a sink (a key of a fixed score without a value: it only adds exp(score) to the softmax's denominator), and an
+// elementwise sigmoid gate on the heads' outputs.
+//
+//   p_j = exp(s_j) / (exp(sink) + sum_i exp(s_i)),   s_j = scale * q . k_j,   max(0, pos - window + 1) <= j <= pos
+//   out = (sum_j p_j v_j) * sigmoid(gate)
+//
+// K is [pages, kv_heads, 64, dim]; V is kept transposed, [pages, kv_heads, vdim, 64].
+//
+// This file: the pass that norms and rotates q and k and writes the step's keys and values to their pages, and the
+// exact kernel (32-bit arithmetic), which serves the float32 mode, single tokens, and whatever the matrix-core kernel
+// does not take.  One block of four waves per (query, group of up to eight query heads that share a key/value head,
+// slice of the key range): a key or value is read once for all those heads.  A wave takes every fourth page of the
+// slice; in a page each lane scores one key for all heads, the wave keeps a running (max, sum, output) for each head,
+// and the four waves' partial results are merged at the end.  With one slice the block then gates and writes the
+// output; with more (a decode step: few queries over long ranges) it leaves its partial result in a workspace for
+// the merging kernel.
+#include "common.h"
+
+constexpr int SK_WAVES = 4;
+constexpr int SK_MAX_DIM = 256;            // of keys and of values
+constexpr int SK_VACC = SK_MAX_DIM / WAVE;
+constexpr int SK_MAX_GROUP = 8;            // query heads a block takes at once
+
+enum SinkNorm : int { SK_NORM_NONE = 0, SK_NORM_PROJECTION = 1, SK_NORM_HEAD = 2 };
+
+// ---- q, k, v of the step's tokens ---------------------------------------------------------------------------
+// One block per token.  The projection-wide sums of squares are made by the whole block; then a wave takes a head
+// (of q or of k) at a time: norm, weight, rotation, and q goes to q_out, k to its page.
+template <typename T>
+__global__ __launch_bounds__(256) void sink_qkv_store_kernel(
+    const T* __restrict__ rows, int stride, int q_off, int k_off, int v_off, const float* __restrict__ bias,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
+    const int* __restrict__ tok_slot, const int* __restrict__ positions, int norm_mode, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+    int heads, int kv_heads, int dim, int vdim, int write_cache) {
+    __shared__ float scratch[16];
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
+    const T* row = rows + t * stride;
+    const int q_size = heads * dim, k_size = kv_heads * dim;
+    const float* q_b = bias, * k_b = bias ? bias + q_size : nullptr, * v_b = bias ? bias + q_size + k_size : nullptr;
+    const int pos = positions[t];
+    const int page = write_cache ? block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS] : 0;
+    const int at = pos % PAGE_TOKENS;
+    float inv_q = 1.f, inv_k = 1.f;
+    if (norm_mode == SK_NORM_PROJECTION) {
+        float sq = 0.f, sk = 0.f;
+        for (int i = threadIdx.x; i < q_size; i += blockDim.x) { const float v = to_float(row[q_off + i]) + (q_b ? q_b[i] : 0.f); sq += v * v; }
+        for (int i = threadIdx.x; i < k_size; i += blockDim.x) { const float v = to_float(row[k_off + i]) + (k_b ? k_b[i] : 0.f); sk += v * v; }
+        sq = block_sum(sq, scratch);
+        sk = block_sum(sk, scratch);
+        inv_q = 1.0f / sqrtf(sq / (float)q_size + eps);
+        inv_k = 1.0f / sqrtf(sk / (float)k_size + eps);
+    }
+    const int half = rot / 2;
+    for (int r = wave; r < heads + kv_heads; r += n_waves) {
+        const bool is_q = r < heads;
+        if (!is_q && !write_cache) continue;
+        const int hh = is_q ? r : r - heads;
+        const T* src = row + (is_q ? q_off : k_off) + (size_t)hh * dim;
+        const float* b = is_q ? (q_b ? q_b + (size_t)hh * dim : nullptr) : (k_b ? k_b + (size_t)hh * dim : nullptr);
+        float inv = is_q ? inv_q : inv_k;
+        const float* w = nullptr;
+        if (norm_mode == SK_NORM_PROJECTION) w = (is_q ? q_w : k_w) + (size_t)hh * dim;
+        if (norm_mode == SK_NORM_HEAD) {
+            w = is_q ? q_w : k_w;
+            float ss = 0.f;
+            for (int d = lane; d < dim; d += WAVE) { const float v = to_float(src[d]) + (b ? b[d] : 0.f); ss += v * v; }
+            inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+        }
+        T* dst = is_q ? q_out + (t * heads + hh) * dim
+                      : k_cache + (((size_t)page * kv_heads + hh) * PAGE_TOKENS + at) * dim;
+        auto normed = [&](int d) {
+            const float v = (to_float(src[d]) + (b ? b[d] : 0.f)) * inv;
+            return w ? v * w[d] : v;
+        };
+        for (int d = lane; d < dim; d += WAVE) {
+            float v = normed(d);
+            if (d < rot) {
+                const int i = d < half ? d : d - half;
+                const float c = cos_t[t * half + i], sn = sin_t[t * half + i];
+                const float pv = normed(d < half ? d + half : d - half);
+                // the pair (u, w) becomes (u c - w s, w c + u s)
+                v = d < half ? v * c - pv * sn : v * c + pv * sn;
+            }
+            dst[d] = from_float<T>(v);
+        }
+    }
+    if (write_cache) {
+        const T* vs = row + v_off;
+        for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x)
+            v_cache[((size_t)page * kv_heads * vdim + i) * PAGE_TOKENS + at] = from_float<T>(to_float(vs[i]) + (v_b ? v_b[i] : 0.f));
+    }
+}
+
+PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype, int stride, int q_off, int k_off, int v_off,
+                                 const float* bias, void* q_out, void* k_cache, void* v_cache, const int* block_table, int max_pages,
+                                 const int* tok_slot, const int* positions, int norm_mode, const float* q_w, const float* k_w, float eps,
+                                 const float* cos_t, const float* sin_t, int rot, int n_tokens, int heads, int kv_heads, int dim, int vdim,
+                                 int write_cache) {
+    PALM_CHECK(n_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "sink_qkv_store: tokens=%d heads=%d kv=%d dim=%d vdim=%d",
+               n_tokens, heads, kv_heads, dim, vdim);
+    PALM_CHECK(norm_mode >= SK_NORM_NONE && norm_mode <= SK_NORM_HEAD, "sink_qkv_store: norm mode %d", norm_mode);
+    PALM_CHECK(norm_mode == SK_NORM_NONE || (q_w && k_w), "sink_qkv_store: a norm needs its weights");
+    PALM_CHECK(rot >= 0 && rot <= dim && rot % 2 == 0, "sink_qkv_store: %d rotated dimensions of %d", rot, dim);
+    PALM_CHECK(rot == 0 || (cos_t && sin_t), "sink_qkv_store: a rotation needs its cos and sin rows");
+    PALM_CHECK(!write_cache || (k_cache && v_cache && block_table && tok_slot && max_pages > 0), "sink_qkv_store: writing needs cache, pages and slots");
+    if (n_tokens == 0) return 0;
+    PALM_DTYPE_SWITCH(dtype, T,
+        sink_qkv_store_kernel<T><<<n_tokens, 256, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
+                                                              (T*)v_cache, block_table, max_pages, tok_slot, positions, norm_mode, q_w, k_w,
+                                                              eps, cos_t, sin_t, rot, heads, kv_heads, dim, vdim, write_cache));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+// ---- the exact kernel -------------------------------------------------------------------------------------
+// 16 bytes of a row at a time where the sizes allow.
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float (&o)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16_t* p, float (&o)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+            o[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+        }
+    }
+};
+
+__device__ inline float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Workspace of a (token, head, slice): m, l, then vdim sums.
+template <typename T, int MAXQ>
+__global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
+    int max_pages, const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_new,
+    const int* __restrict__ cu_new, int heads, int kv_heads, int dim, int vdim, float scale, int window, int has_sink,
+    float sink_score, const T* __restrict__ gate, int gate_stride, int n_slices, float* __restrict__ work, T* __restrict__ out) {
+    __shared__ float q_s[MAXQ][SK_MAX_DIM];
+    __shared__ float m_s[SK_WAVES][MAXQ], l_s[SK_WAVES][MAXQ];
+    __shared__ float acc_s[SK_WAVES][MAXQ][SK_MAX_DIM];
+
+    const int per_kv = heads / kv_heads;
+    const int chunks = (per_kv + MAXQ - 1) / MAXQ;                 // a group of more than MAXQ heads goes through in several blocks
+    const int qi = blockIdx.x, g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int b = blockIdx.z / n_slices, slice = blockIdx.z % n_slices;
+    if (qi >= seq_new[b]) return;
+    const int h0 = g * per_kv + chunk * MAXQ;
+    const int nq = min(MAXQ, per_kv - chunk * MAXQ);
+    const int t = cu_new[b] + qi;
+    const int pos = seq_start[b] + qi;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
+
+    for (int i = threadIdx.x; i < MAXQ * dim; i += blockDim.x) {
+        const int qh = i / dim, d = i % dim;
+        q_s[qh][d] = qh < nq ? to_float(q[((size_t)t * heads + h0 + qh) * dim + d]) * scale : 0.f;
+    }
+    __syncthreads();
+
+    float m[MAXQ], l[MAXQ], acc[MAXQ][SK_VACC];
+#pragma unroll
+    for (int qh = 0; qh < MAXQ; ++qh) {
+        const bool sink_here = has_sink && slice == 0 && wave == 0;
+        m[qh] = sink_here ? sink_score : -INFINITY;
+        l[qh] = sink_here ? 1.f : 0.f;
+#pragma unroll
+        for (int i = 0; i < SK_VACC; ++i) acc[qh][i] = 0.f;
+    }
+
+    // this slice's pages
+    const int p_lo = lo / PAGE_TOKENS, p_hi = pos / PAGE_TOKENS;
+    const int per_slice = (p_hi - p_lo + n_slices) / n_slices;
+    const int s_lo = p_lo + slice * per_slice, s_hi = min(p_hi, s_lo + per_slice - 1);
+    constexpr int VN = Vec16<T>::N;
+    const bool k_vec = dim % VN == 0;
+
+    for (int pg = s_lo + wave; pg <= s_hi; pg += SK_WAVES) {
+        const int page = pages[pg];
+        const T* kp = k_cache + ((size_t)page * kv_heads + g) * PAGE_TOKENS * dim;
+        const T* vp = v_cache + ((size_t)page * kv_heads + g) * (size_t)vdim * PAGE_TOKENS;
+        const int j = pg * PAGE_TOKENS + lane;
+        const bool seen = j >= lo && j <= pos;
+        float s[MAXQ];
+#pragma unroll
+        for (int qh = 0; qh < MAXQ; ++qh) s[qh] = 0.f;
+        const T* kr = kp + (size_t)lane * dim;
+        if (k_vec) {
+            for (int d0 = 0; d0 < dim; d0 += VN) {
+                float kv[VN];
+                Vec16<T>::load(kr + d0, kv);
+#pragma unroll
+                for (int e = 0; e < VN; ++e)
+#pragma unroll
+                    for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d0 + e], kv[e], s[qh]);
+            }
+        } else {
+            for (int d = 0; d < dim; ++d) {
+                const float kd = to_float(kr[d]);
+#pragma unroll
+                for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d], kd, s[qh]);
+            }
+        }
+        float p[MAXQ];
+#pragma unroll
+        for (int qh = 0; qh < MAXQ; ++qh) {
+            const float sc = seen ? s[qh] : -INFINITY;
+            const float m_new = fmaxf(m[qh], wave_max(sc));       // every page of the range holds a key that is seen
+            const float alpha = expf(m[qh] - m_new);              // m = -inf at the first page: exp(-inf) = 0
+            p[qh] = expf(sc - m_new);                             // a key that is not seen: exp(-inf) = 0
+            l[qh] = l[qh] * alpha + wave_sum(p[qh]);
+            m[qh] = m_new;
+#pragma unroll
+            for (int i = 0; i < SK_VACC; ++i) acc[qh][i] *= alpha;
+        }
+        // values: lane c owns columns c, c + 64, ..; its rows of the transposed page are read 16 bytes at a time
+        const int j_first = max(lo, pg * PAGE_TOKENS) - pg * PAGE_TOKENS;
+        const int j_last = min(pos, pg * PAGE_TOKENS + PAGE_TOKENS - 1) - pg * PAGE_TOKENS;
+        for (int j0 = j_first / VN * VN; j0 <= j_last; j0 += VN) {
+            float vv[SK_VACC][VN];
+#pragma unroll
+            for (int i = 0; i < SK_VACC; ++i) {
+                const int c = min(lane + i * WAVE, vdim - 1);
+                if (i * WAVE < vdim) Vec16<T>::load(vp + (size_t)c * PAGE_TOKENS + j0, vv[i]);
+            }
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+#pragma unroll
+                for (int qh = 0; qh < MAXQ; ++qh) {
+                    const float pj = lane_value(p[qh], j0 + e);   // zero for a key that is not seen
+#pragma unroll
+                    for (int i = 0; i < SK_VACC; ++i)
+                        if (i * WAVE < vdim) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int qh = 0; qh < MAXQ; ++qh) {
+        if (lane == 0) { m_s[wave][qh] = m[qh]; l_s[wave][qh] = l[qh]; }
+#pragma unroll
+        for (int i = 0; i < SK_VACC; ++i) {
+            const int c = lane + i * WAVE;
+            if (c < vdim) acc_s[wave][qh][c] = acc[qh][i];
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nq * vdim; i += blockDim.x) {
+        const int qh = i / vdim, c = i % vdim, h = h0 + qh;
+        float m_all = -INFINITY;
+        for (int w = 0; w < SK_WAVES; ++w) m_all = fmaxf(m_all, m_s[w][qh]);
+        float l_all = 0.f, o = 0.f;
+        for (int w = 0; w < SK_WAVES; ++w) {
+            const float f = m_s[w][qh] == -INFINITY ? 0.f : expf(m_s[w][qh] - m_all);
+            l_all += l_s[w][qh] * f;
+            o += acc_s[w][qh][c] * f;
+        }
+        if (n_slices == 1) {
+            float r = o / l_all;
+            if (gate) { const float gt = to_float(gate[(size_t)t * gate_stride + (size_t)h * vdim + c]); r *= 1.0f / (1.0f + expf(-gt)); }
+            out[((size_t)t * heads + h) * vdim + c] = from_float<T>(r);
+        } else {
+            float* wk = work + (((size_t)t * heads + h) * n_slices + slice) * (vdim + 2);
+            if (c == 0) { wk[0] = m_all; wk[1] = l_all; }
+            wk[2 + c] = o;
+        }
+    }
+}
+
+// The slices of a (token, head) merged, gated and written.
+template <typename T>
+__global__ void sink_attention_merge_kernel(const float* __restrict__ work, int n_slices, int heads, int vdim, const T* __restrict__ gate,
+                                            int gate_stride, T* __restrict__ out) {
+    const size_t t = blockIdx.x;
+    const int h = blockIdx.y;
+    const float* wk = work + ((t * heads + h) * n_slices) * (size_t)(vdim + 2);
+    float m_all = -INFINITY;
+    for (int s = 0; s < n_slices; ++s) m_all = fmaxf(m_all, wk[(size_t)s * (vdim + 2)]);
+    float l_all = 0.f;
+    for (int s = 0; s < n_slices; ++s) {
+        const float ms = wk[(size_t)s * (vdim + 2)];
+        l_all += ms == -INFINITY ? 0.f : wk[(size_t)s * (vdim + 2) + 1] * expf(ms - m_all);
+    }
+    for (int c = threadIdx.x; c < vdim; c += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < n_slices; ++s) {
+            const float ms = wk[(size_t)s * (vdim + 2)];
+            if (ms != -INFINITY) o += wk[(size_t)s * (vdim + 2) + 2 + c] * expf(ms - m_all);
+        }
+        float r = o / l_all;
+        if (gate) { const float gt = to_float(gate[t * gate_stride + (size_t)h * vdim + c]); r *= 1.0f / (1.0f + expf(-gt)); }
+        out[(t * heads + h) * vdim + c] = from_float<T>(r);
+    }
+}
+
+// q [n, heads, dim]; gate: null, or the first gate value of token 0 (rows `gate_stride` elements apart, heads * vdim
+// values a row); work: room for n_tokens * heads * n_slices * (vdim + 2) floats if n_slices > 1; out [n, heads * vdim].
+PALM_API int palm_sink_attention(hipStream_t stream, const void* q, int dtype, const void* k_cache, const void* v_cache,
+                                 const int* block_table, int max_pages, const int* seq_slot, const int* seq_start, const int* seq_new,
+                                 const int* cu_new, int n_seqs, int max_new, int n_tokens, int heads, int kv_heads, int dim, int vdim,
+                                 float scale, int window, int has_sink, float sink_score, const void* gate, int gate_stride, int n_slices,
+                                 float* work, void* out) {
+    PALM_CHECK(n_seqs >= 0 && max_new >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0,
+               "sink_attention: seqs=%d max_new=%d heads=%d kv=%d dim=%d vdim=%d", n_seqs, max_new, heads, kv_heads, dim, vdim);
+    PALM_CHECK(heads % kv_heads == 0, "sink_attention: %d heads are not a multiple of %d kv heads", heads, kv_heads);
+    PALM_CHECK(dim <= SK_MAX_DIM && vdim <= SK_MAX_DIM, "sink_attention: key size %d / value size %d exceed %d", dim, vdim, SK_MAX_DIM);
+    PALM_CHECK(window >= 0 && max_pages > 0, "sink_attention: window %d, max_pages %d", window, max_pages);
+    PALM_CHECK(n_slices >= 1 && (n_slices == 1 || work), "sink_attention: %d slices need a workspace", n_slices);
+    if (n_seqs == 0 || max_new == 0 || n_tokens == 0) return 0;
+    const int per_kv = heads / kv_heads;
+    const int maxq = per_kv >= 8 ? 8 : per_kv > 2 ? 4 : per_kv;
+    const int chunks = (per_kv + maxq - 1) / maxq;
+    PALM_CHECK(kv_heads * chunks <= 65535 && (long long)n_seqs * n_slices <= 65535,
+               "sink_attention: %d kv heads / %d sequences x %d slices are more than one launch takes", kv_heads, n_seqs, n_slices);
+    dim3 grid(max_new, kv_heads * chunks, n_seqs * n_slices);
+#define SK_CASE(Q) sink_attention_kernel<T, Q><<<grid, SK_WAVES * WAVE, 0, stream>>>((const T*)q, (const T*)k_cache, (const T*)v_cache, \
+        block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, heads, kv_heads, dim, vdim, scale, window, has_sink, sink_score, \
+        (const T*)gate, gate_stride, n_slices, work, (T*)out)
+    PALM_DTYPE_SWITCH(dtype, T, {
+        if (maxq == 1) SK_CASE(1); else if (maxq == 2) SK_CASE(2); else if (maxq == 4) SK_CASE(4); else SK_CASE(8);
+        if (n_slices > 1)
+            sink_attention_merge_kernel<T><<<dim3(n_tokens, heads), 64, 0, stream>>>(work, n_slices, heads, vdim, (const T*)gate, gate_stride,
+                                                                                    (T*)out);
+    });
+#undef SK_CASE
+    PALM_LAUNCHED();
+    return 0;
+}
+
+PALM_DEFINE_LAST_ERROR()

@@ -7,6 +7,11 @@
 // q and k are rotated first (pairs (i, i + rot/2) of the first `rot` dimensions, cos/sin rows of the tokens'
 // positions) and k is multiplied by k_scale after the rotation; rotated values, state and sums are 32-bit.
 //
+// Two options make this the recurrence of other linear attentions as well: `act` puts q, k and v through silu first
+// (q and k before the rotation), and `joined` leaves out the per-head unit norm and the gate: the heads' o_t are then
+// written as they are, 32-bit, and a pass of its own norms a token's joined heads together, with a weight, and gates
+// them (palm_joined_norm_gate).
+//
 // A first pass rotates q and k of all the step's tokens into 32-bit rows.  Then one block per (head, sequence), one
 // thread per value dimension v: the thread keeps column v of S in registers and walks over the sequence's new
 // tokens.  A token's rotated q and k are the same for every thread of the block: each wave reads the two rows once,
@@ -26,13 +31,15 @@ constexpr int RET_TILE = 8;
 
 enum RetentionMode : int { RET_WHOLE = 0, RET_LOCAL = 1, RET_FROM_STARTS = 2 };
 
+__device__ inline float ret_silu(float z) { return z / (1.0f + expf(-z)); }
+
 // q and k of every token and head, rotated (k also scaled), 32-bit: qk[row][head][0 = q, 1 = k][pad], pad >= dim the
 // key size that the main kernel is compiled for; the columns beyond dim are zero, so that the main kernel's loops
 // over pad need no test (a zero k leaves its row of S zero, a zero q adds nothing).
 template <typename T>
 __global__ void retention_rotate_kernel(const T* __restrict__ qkvg, int row_stride, int q_off, int k_off,
                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, float k_scale,
-                                        int n_tokens, int heads, int dim, int pad, float* __restrict__ qk) {
+                                        int act, int n_tokens, int heads, int dim, int pad, float* __restrict__ qk) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long long)n_tokens * heads * pad) return;
     const int d = (int)(idx % pad), h = (int)((idx / pad) % heads);
@@ -43,11 +50,13 @@ __global__ void retention_rotate_kernel(const T* __restrict__ qkvg, int row_stri
     const T* qr = qkvg + row * row_stride + q_off + h * dim;
     const T* kr = qkvg + row * row_stride + k_off + h * dim;
     float qv = to_float(qr[d]), kv = to_float(kr[d]);
+    if (act) { qv = ret_silu(qv); kv = ret_silu(kv); }
     if (d < rot) {
         const int i = d < half ? d : d - half;
         const float c = cos_t[row * half + i], sn = sin_t[row * half + i];
         const int partner = d < half ? d + half : d - half;
-        const float qp = to_float(qr[partner]), kp = to_float(kr[partner]);
+        float qp = to_float(qr[partner]), kp = to_float(kr[partner]);
+        if (act) { qp = ret_silu(qp); kp = ret_silu(kp); }
         // the pair (u, w) becomes (u c - w s, w c + u s)
         qv = d < half ? qv * c - qp * sn : qv * c + qp * sn;
         kv = d < half ? kv * c - kp * sn : kv * c + kp * sn;
@@ -64,7 +73,7 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
                                  const float* __restrict__ decay, float eps,
                                  float* __restrict__ state, const int* __restrict__ seq_slot,
                                  const int* __restrict__ seq_new, const int* __restrict__ cu_new,
-                                 int heads, int dim, int vdim, T* __restrict__ out) {
+                                 int heads, int dim, int vdim, T* __restrict__ out, int act, int joined, float* __restrict__ raw) {
     __shared__ float red[RET_TILE][16];
     __shared__ float o_s[RET_TILE][MAXT];
     constexpr int QREGS = (DMAX + WAVE - 1) / WAVE;
@@ -100,6 +109,7 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
     auto read_token = [&](int t, float& vv, float (&qv)[QREGS], float (&kv)[QREGS]) {
         const size_t row = (size_t)(row0 + t);
         vv = to_float(qkvg[row * row_stride + v_off + h * vdim + vc]);
+        if (act) vv = ret_silu(vv);
         const float* __restrict__ qr = qk + ((row * heads + h) * 2) * DMAX;
 #pragma unroll
         for (int c = 0; c < QREGS; ++c) {
@@ -124,7 +134,9 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
                 S[d] = fmaf(g, S[d], kd * vv);
                 acc = fmaf(S[d], qd, acc);
             }
-            if (mode != RET_LOCAL) {
+            if (mode != RET_LOCAL && joined) {
+                if (mine) raw[(size_t)(row0 + t0 + ti) * ((size_t)heads * vdim) + h * vdim + v] = acc;
+            } else if (mode != RET_LOCAL) {
                 o_s[ti][v] = acc;
                 const float ss = wave_sum(acc * acc);
                 if (lane == 0) red[ti][wave] = ss;
@@ -133,7 +145,7 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
 #pragma unroll
             for (int c = 0; c < QREGS; ++c) { qv[c] = qn[c]; kv[c] = kn[c]; }
         }
-        if (mode == RET_LOCAL) continue;
+        if (mode == RET_LOCAL || joined) continue;
         __syncthreads();
         for (int ti = 0; ti < tt; ++ti) {
             float total = 0.f;
@@ -176,11 +188,11 @@ template <typename T>
 static void retention_launch(hipStream_t stream, dim3 grid, int threads, int mode, int chunk, int max_chunks, float* starts,
                              const T* qkvg, int row_stride, int v_off, int g_off, const float* qk, const float* decay,
                              float eps, float* state, const int* seq_slot, const int* seq_new,
-                             const int* cu_new, int heads, int dim, int vdim, T* out) {
+                             const int* cu_new, int heads, int dim, int vdim, T* out, int act, int joined, float* raw) {
 #define RET_CASE(D) { if (threads <= 256) retention_kernel<T, D, 256><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, \
-            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out); \
+            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out, act, joined, raw); \
         else retention_kernel<T, D, 1024><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, \
-            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out); }
+            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out, act, joined, raw); }
     if (dim <= 32) RET_CASE(32)
     else if (dim <= 64) RET_CASE(64)
     else if (dim <= 128) RET_CASE(128)
@@ -196,7 +208,7 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
                             int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay, float k_scale,
                             float eps, float* state, const int* seq_slot, const int* seq_new, const int* cu_new, int n_seqs,
                             int heads, int dim, int vdim, void* out, int max_new, int chunk, float* starts, int n_tokens,
-                            float* qk) {
+                            float* qk, int act, int joined, float* raw) {
     PALM_CHECK(n_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0, "retention: seqs=%d heads=%d dim=%d vdim=%d", n_seqs, heads, dim, vdim);
     PALM_CHECK(dim <= 256, "retention: a key size of %d exceeds 256", dim);
     PALM_CHECK(vdim <= 1024, "retention: a value size of %d exceeds 1024", vdim);
@@ -204,6 +216,7 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "retention: a rotation needs its cos and sin rows");
     PALM_CHECK(chunk >= 0 && (chunk == 0 || (starts && max_new > 0)), "retention: chunks of %d tokens need their starting states", chunk);
     PALM_CHECK(n_tokens >= 0 && (n_tokens == 0 || qk), "retention: the rotated q and k need their room");
+    PALM_CHECK(n_tokens == 0 || (joined ? raw != nullptr : out != nullptr), "retention: the outputs need their room (32-bit rows if the heads are normed together later)");
     if (n_seqs == 0 || n_tokens == 0) return 0;
     const int max_chunks = chunk > 0 ? (max_new + chunk - 1) / chunk : 1;
     PALM_CHECK(heads <= 65535 && (long long)n_seqs * max_chunks <= 65535, "retention: %d heads / %d sequences x %d chunks are more than one launch takes",
@@ -214,20 +227,54 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
     const long long rot_threads = (long long)n_tokens * heads * pad;
     PALM_DTYPE_SWITCH(dtype, T, {
         retention_rotate_kernel<T><<<(unsigned)((rot_threads + 255) / 256), 256, 0, stream>>>((const T*)qkvg, row_stride, q_off, k_off, cos_t,
-                                                                                             sin_t, rot, k_scale, n_tokens, heads, dim, pad, qk);
+                                                                                             sin_t, rot, k_scale, act, n_tokens, heads, dim, pad, qk);
         if (chunk == 0) {
             retention_launch<T>(stream, grid, threads, RET_WHOLE, 1 << 30, 1, nullptr, (const T*)qkvg, row_stride, v_off, g_off, qk, decay,
-                                eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+                                eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out, act, joined, raw);
         } else {
             retention_launch<T>(stream, grid, threads, RET_LOCAL, chunk, max_chunks, starts, (const T*)qkvg, row_stride, v_off, g_off, qk,
-                                decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+                                decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out, act, joined, raw);
             const int elems = heads * dim * vdim;
             retention_starts_kernel<<<dim3((elems + 255) / 256, n_seqs), 256, 0, stream>>>(starts, state, decay, seq_slot, seq_new, chunk,
                                                                                          max_chunks, heads, dim * vdim);
             retention_launch<T>(stream, grid, threads, RET_FROM_STARTS, chunk, max_chunks, starts, (const T*)qkvg, row_stride, v_off, g_off,
-                                qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+                                qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out, act, joined, raw);
         }
     });
     PALM_LAUNCHED();
     return 0;
 }
+
+// ---- the joined heads normed together and gated -------------------------------------------------------------
+// out[t] = raw[t] / sqrt(mean(raw[t]^2) + eps) * weight * f(gate[t]) over a token's whole row of `width` values (all
+// heads), f = sigmoid (gate_act 1) or silu (gate_act 0).  raw is 32-bit; the gate lies in rows `gate_stride` elements
+// apart.  One block per token.
+template <typename T>
+__global__ __launch_bounds__(256) void joined_norm_gate_kernel(const float* __restrict__ raw, const float* __restrict__ weight, float eps,
+                                                               const T* __restrict__ gate, int gate_stride, int gate_act, int width,
+                                                               T* __restrict__ out) {
+    __shared__ float scratch[16];
+    const size_t t = blockIdx.x;
+    const float* r = raw + t * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) { const float v = r[c]; ss += v * v; }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float g = to_float(gate[t * gate_stride + c]);
+        const float f = gate_act == 1 ? 1.0f / (1.0f + expf(-g)) : g / (1.0f + expf(-g));
+        out[t * width + c] = from_float<T>(r[c] * inv * weight[c] * f);
+    }
+}
+
+PALM_API int palm_joined_norm_gate(hipStream_t stream, const float* raw, const float* weight, float eps, const void* gate, int dtype,
+                                   int gate_stride, int gate_act, int n_tokens, int width, void* out) {
+    PALM_CHECK(n_tokens >= 0 && width > 0 && gate_stride >= width, "joined_norm_gate: tokens=%d width=%d gate rows %d apart", n_tokens, width, gate_stride);
+    PALM_CHECK(gate_act == 0 || gate_act == 1, "joined_norm_gate: gate activation %d is neither silu (0) nor sigmoid (1)", gate_act);
+    if (n_tokens == 0) return 0;
+    PALM_DTYPE_SWITCH(dtype, T,
+        joined_norm_gate_kernel<T><<<n_tokens, 256, 0, stream>>>(raw, weight, eps, (const T*)gate, gate_stride, gate_act, width, (T*)out));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+PALM_DEFINE_LAST_ERROR()

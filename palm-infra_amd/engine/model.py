@@ -56,9 +56,14 @@ class DecoderModel:
             return self.head.forward(self.final_norm(x, rows=want_rows))
         # a layer gets its first norm's output and returns the output of the norm after it: the next layer's
         # first norm, at the end the final norm over the wanted rows
+        # entries that add the embedding's rows again need them as they left the embedding
+        x0 = x.clone() if any(call.adds_embedding for call in self.order) else None
         h = self.layers[self.order[0].layer].entry_norm(x)
         for i, call in enumerate(self.order):
             ctx.layer_cache = cache.layer_caches[i]
+            if call.adds_embedding:
+                # the sum is made in 32-bit in the pass that norms it for this entry
+                h = self.layers[call.layer].entry_norm(x, delta=x0, update=True)
             if i + 1 < len(self.order):
                 sink = ResidualSink(x, self.layers[self.order[i + 1].layer].entry_norm)
             else:

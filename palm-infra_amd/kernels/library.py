@@ -9,7 +9,13 @@ built or loaded, the error says so and nothing runs.
 Libraries:
   ``core``              every kernel that does not depend on the head size
   ``attention_hd<N>``   the matrix-core attention kernels, compiled for one head size
-  ``mixers``            the mixers beside softmax attention over equal key and value sizes (retention, the selective
+  ``recurrent``         linear attention with one fixed decay per head (retention), with its options
+  ``sink_attention``    softmax attention with a sink, a window, a gate and key and value sizes of their own: the pass that
+                        prepares q, k and v, and the exact kernel
+  ``sink_attention_k<K>_v<V>``  the same attention for prompts on the matrix cores, compiled for key sizes up to 32 K and
+                        value sizes up to 16 V
+  ``branches``          branch outputs scaled by a learned vector into the residual stream; the capped feed-forward gate
+  ``mixers``            the other mixers beside softmax attention over equal key and value sizes (the selective
                         scan and its convolution, differential attention, the delta rule, attention over compressed
                         rows), routed experts, and the stream of blocks that norm a branch's output; loaded when a
                         model has such a part
@@ -48,8 +54,12 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
 ATTENTION_SOURCES = ["attention_mfma.hip"]
 DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
 LATENT_ATTENTION_SOURCES = ["latent_attention_mfma.hip"]
-MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
+MIXER_SOURCES = ["stream.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
                  "latent_attention.hip", "moe.hip", "moe_grouped.hip"]
+RECURRENT_SOURCES = ["retention.hip"]
+SINK_ATTENTION_SOURCES = ["attention_sink.hip"]
+SINK_ATTENTION_MFMA_SOURCES = ["attention_sink_mfma.hip"]
+BRANCH_SOURCES = ["branch_scaled.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
 
@@ -177,6 +187,15 @@ def _spec(name: str):
         return CORE_SOURCES, ()
     if name == "mixers":
         return MIXER_SOURCES, ()
+    if name == "recurrent":
+        return RECURRENT_SOURCES, ()
+    if name == "sink_attention":
+        return SINK_ATTENTION_SOURCES, ()
+    if name == "branches":
+        return BRANCH_SOURCES, ()
+    if name.startswith("sink_attention_k"):
+        kk, vt = name[len("sink_attention_k"):].split("_v")
+        return SINK_ATTENTION_MFMA_SOURCES, (f"PALM_SINK_KK={int(kk)}", f"PALM_SINK_VT={int(vt)}")
     if name.startswith("attention_diff_k"):
         kk, rest = name[len("attention_diff_k"):].split("_v")
         vt, qt = rest.split("_q")

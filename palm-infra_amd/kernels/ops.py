@@ -762,10 +762,6 @@ _MIXER_SIGNATURES = {
     "palm_add_normed": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p, c_int,
                         c_longlong, c_void_p, c_int],
     "palm_xielu": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_longlong],
-    "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
-                       c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
-                       c_void_p, c_int, c_void_p],
-    "palm_retention_pad": [c_int],
     "palm_causal_conv": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_void_p],
     "palm_selective_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -810,6 +806,53 @@ def mixers():
             fn.argtypes, fn.restype = argtypes, c_int
         _mixers = lib
     return _mixers
+
+
+_RECURRENT_SIGNATURES = {
+    "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                       c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
+                       c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "palm_retention_pad": [c_int],
+    "palm_joined_norm_gate": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+}
+_SINK_SIGNATURES = {
+    "palm_sink_qkv_store": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                            c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                            c_int, c_int, c_int],
+    "palm_sink_attention": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_int, c_int,
+                            c_void_p, c_void_p],
+}
+_BRANCH_SIGNATURES = {
+    "palm_add_scaled_normed": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_int, c_void_p, c_void_p, c_float, c_void_p,
+                               c_int, c_int, c_int, c_void_p, c_int],
+    "palm_capped_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_float],
+}
+_small_libraries: dict = {}
+
+
+def _small(name: str, signatures: dict):
+    """A library of one mechanism, loaded (and built, if it never was) when a model first uses the mechanism."""
+    lib = _small_libraries.get(name)
+    if lib is None:
+        lib = library.load(name)
+        for fn_name, argtypes in signatures.items():
+            fn = getattr(lib, fn_name)
+            fn.argtypes, fn.restype = argtypes, c_int
+        _small_libraries[name] = lib
+    return lib
+
+
+def recurrent():
+    return _small("recurrent", _RECURRENT_SIGNATURES)
+
+
+def sink_attention_lib():
+    return _small("sink_attention", _SINK_SIGNATURES)
+
+
+def branches():
+    return _small("branches", _BRANCH_SIGNATURES)
 
 
 def add_normed(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
@@ -865,10 +908,15 @@ def retention_chunk(n_seqs: int, heads: int, max_new: int) -> int:
 
 
 def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, k_scale: float, eps: float,
-              state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0, chunk: int | None = None) -> torch.Tensor:
+              state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0, chunk: int | None = None, input_silu: bool = False,
+              joined_norm: torch.Tensor | None = None, gate_sigmoid: bool = False) -> torch.Tensor:
     """The step's tokens through a retention layer's recurrence.  qkvg [n, heads * (2 dim + 2 vdim)] holds q | k | v |
     gate; state float32 [slots, heads, dim, vdim] is read and left updated.  Returns [n, heads * vdim]: the heads'
-    outputs, unit-normed per head and gated.  ``chunk``: see ``retention_chunk`` (None: chosen here)."""
+    outputs, unit-normed per head and gated by silu of the gate.  ``chunk``: see ``retention_chunk`` (None: chosen here).
+
+    ``input_silu``: q, k and v go through silu first.  ``joined_norm`` (float32 [heads * vdim]): instead of the unit norm
+    per head, a token's joined heads are normed together and multiplied by this weight; ``gate_sigmoid``: the gate is then
+    sigmoid of the gate values instead of silu."""
     _dev("retention", qkvg, decay, state, cos, sin, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     _i32("retention", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     n = qkvg.shape[0]
@@ -882,17 +930,29 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
         for tab in (cos, sin):
             _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"retention: rotation rows are float32 [{n}, {rot // 2}]")
     out = torch.empty((n, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    raw = None
+    if joined_norm is not None:
+        _dev("retention", joined_norm)
+        _need(joined_norm.shape == (heads * vdim,) and joined_norm.dtype == F32, f"retention: the joined heads' norm weight is float32 [{heads * vdim}]")
+        raw = torch.empty((n, heads * vdim), dtype=F32, device=qkvg.device)
+    else:
+        _need(not gate_sigmoid, "retention: the per-head unit norm comes with a silu gate")
     chunk = retention_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
     # q and k after the rotation, 32-bit, in rows padded to the key size that the kernel is compiled for
-    rotated = torch.empty((n, heads, 2, mixers().palm_retention_pad(dim)), dtype=F32, device=qkvg.device)
+    rotated = torch.empty((n, heads, 2, recurrent().palm_retention_pad(dim)), dtype=F32, device=qkvg.device)
     starts = None
     if chunk:
         max_chunks = -(-ctx.max_new // chunk)
         starts = torch.empty((ctx.n_seqs * max_chunks, heads, dim, vdim), dtype=F32, device=qkvg.device)
-    library.call(mixers(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
-                 2 * heads * dim, 2 * heads * dim + heads * vdim, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
+    g_off = 2 * heads * dim + heads * vdim
+    library.call(recurrent(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
+                 2 * heads * dim, g_off, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
                  _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out),
-                 int(ctx.max_new), chunk, _p(starts), n, _p(rotated))
+                 int(ctx.max_new), chunk, _p(starts), n, _p(rotated), int(input_silu), int(raw is not None), _p(raw))
+    if raw is not None:
+        library.call(recurrent(), "palm_joined_norm_gate", _stream(), _p(raw), _p(joined_norm), float(eps),
+                     qkvg.data_ptr() + g_off * qkvg.element_size(), _code(qkvg, "retention"), qkvg.shape[1], int(gate_sigmoid), n,
+                     heads * vdim, _p(out))
     return out
 
 
@@ -1380,3 +1440,124 @@ def scatter_add(out: torch.Tensor, y: torch.Tensor, rows: torch.Tensor, weight: 
           and weight.shape == (y.shape[0],) and weight.dtype == F32, f"scatter_add: out {tuple(out.shape)} {out.dtype}, y {tuple(y.shape)}, "
           f"rows {tuple(rows.shape)}, weights {tuple(weight.shape)} {weight.dtype}")
     library.call(mixers(), "palm_scatter_add", _stream(), _p(y), _code(y, "scatter_add"), _p(rows), _p(weight), y.shape[0], out.shape[1], _p(out))
+
+
+# ---- softmax attention with a sink, a window and a gate (library ``sink_attention``) -------------------------------
+
+SINK_NORMS = {None: 0, "projection": 1, "head": 2}
+SINK_BLOCKS_WANTED = 1024         # a decode step's key ranges are cut into slices until about this many blocks run
+
+
+def sink_qkv_store(rows: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, bias, norm: str | None, q_w, k_w, eps: float,
+                   cos, sin, rot: int, k_cache, v_cache, block_table, ctx, write_cache: bool = True) -> torch.Tensor:
+    """q, k and v of the step's tokens from ``rows`` [n, >= heads*dim + kv_heads*dim + kv_heads*vdim] (q | k | v | whatever
+    follows): ``bias`` (float32 over q | k | v, or None) is added, q and k are normed (``norm``: "projection": one RMS norm
+    over the whole q row and one over the whole k row, weights of those sizes; "head": per head, weights of the key size;
+    None), their first ``rot`` dimensions are rotated by the tokens' cos and sin rows, k and v go to their pages, and q
+    comes back as [n, heads, dim]."""
+    _dev("sink_qkv_store", rows, bias, q_w, k_w, cos, sin, k_cache, v_cache, block_table, ctx.tok_slot, ctx.positions)
+    _i32("sink_qkv_store", block_table, ctx.tok_slot, ctx.positions)
+    n = rows.shape[0]
+    q_size, k_size, v_size = heads * dim, kv_heads * dim, kv_heads * vdim
+    _need(rows.dim() == 2 and rows.shape[1] >= q_size + k_size + v_size and n == ctx.n_tokens,
+          f"sink_qkv_store: rows {tuple(rows.shape)} for {ctx.n_tokens} tokens of {q_size} + {k_size} + {v_size}")
+    _need(norm in SINK_NORMS, f"sink_qkv_store: norm {norm!r} is not one of {sorted(map(str, SINK_NORMS))}")
+    if bias is not None:
+        _need(bias.shape == (q_size + k_size + v_size,) and bias.dtype == F32, f"sink_qkv_store: the bias is float32 [{q_size + k_size + v_size}]")
+    if norm is not None:
+        want = (q_size, k_size) if norm == "projection" else (dim, dim)
+        _need(q_w is not None and k_w is not None and q_w.shape == (want[0],) and k_w.shape == (want[1],) and q_w.dtype == F32
+              and k_w.dtype == F32, f"sink_qkv_store: the norm weights are float32 [{want[0]}] and [{want[1]}]")
+    if rot:
+        for tab in (cos, sin):
+            _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"sink_qkv_store: rotation rows are float32 [{n}, {rot // 2}]")
+    _need(k_cache.dtype == rows.dtype and v_cache.dtype == rows.dtype and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
+          and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS) and block_table.dim() == 2,
+          f"sink_qkv_store: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} for rows of {rows.dtype}")
+    q = torch.empty((n, heads, dim), dtype=rows.dtype, device=rows.device)
+    library.call(sink_attention_lib(), "palm_sink_qkv_store", _stream(), _p(rows), _code(rows, "sink_qkv_store"), rows.shape[1], 0, q_size,
+                 q_size + k_size, _p(bias), _p(q), _p(k_cache), _p(v_cache), _p(block_table), block_table.shape[1], _p(ctx.tok_slot),
+                 _p(ctx.positions), SINK_NORMS[norm], _p(q_w), _p(k_w), float(eps), _p(cos), _p(sin), int(rot), n, heads, kv_heads, dim,
+                 vdim, int(write_cache))
+    return q
+
+
+def sink_slices(ctx, heads: int, kv_heads: int, window: int | None) -> int:
+    """Into how many slices the exact kernel cuts a query's key range: one for prompts; for single tokens as many as
+    fill the chip, each of at least four pages (a block's four waves take a page each)."""
+    if not ctx.is_decode:
+        return 1
+    keys = min(ctx.max_total, window) if window else ctx.max_total
+    pages = -(-keys // PAGE_TOKENS) + 1
+    blocks = ctx.n_seqs * kv_heads * -(-(heads // kv_heads) // 8)
+    return max(1, min(pages // 4, SINK_BLOCKS_WANTED // max(1, blocks)))
+
+
+def sink_attention_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
+                         scale: float, window: int | None, sink: float | None, gate: torch.Tensor | None, gate_off: int = 0,
+                         slices: int | None = None) -> torch.Tensor:
+    """Attention of the step's queries q [n, heads, dim] over the cached keys of their sequences up to their own positions
+    (the last ``window`` if given), with a sink of score ``sink`` (None: none) in the denominator.  ``gate``: a tensor [n,
+    >= gate_off + heads*vdim] whose columns from ``gate_off`` on gate the output through a sigmoid (None: no gate).  Returns
+    [n, heads * vdim].  32-bit arithmetic whatever the elements' type."""
+    _dev("sink_attention", q, k_cache, v_cache, block_table, gate, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _i32("sink_attention", block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    n = q.shape[0]
+    _need(q.shape == (ctx.n_tokens, heads, dim), f"sink_attention: q {tuple(q.shape)} is not [{ctx.n_tokens}, {heads}, {dim}]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
+          and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS), f"sink_attention: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= gate_off + heads * vdim and gate.dtype == q.dtype,
+              f"sink_attention: gate rows {tuple(gate.shape)} {gate.dtype} from column {gate_off}")
+        gate_ptr, gate_stride = gate.data_ptr() + gate_off * gate.element_size(), gate.shape[1]
+    slices = sink_slices(ctx, heads, kv_heads, window) if slices is None else int(slices)
+    work = torch.empty((n * heads * slices * (vdim + 2),), dtype=F32, device=q.device) if slices > 1 else None
+    out = torch.empty((n, heads * vdim), dtype=q.dtype, device=q.device)
+    library.call(sink_attention_lib(), "palm_sink_attention", _stream(), _p(q), _code(q, "sink_attention"), _p(k_cache), _p(v_cache),
+                 _p(block_table), block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs,
+                 int(ctx.max_new), n, heads, kv_heads, dim, vdim, float(scale), int(window or 0), int(sink is not None),
+                 float(sink or 0.0), gate_ptr, gate_stride, slices, _p(work), _p(out))
+    return out
+
+
+def sink_attention(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off=0):
+    """The kernel that serves: the exact one for the float32 mode and for single tokens."""
+    return sink_attention_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off)
+
+
+# ---- branches scaled by a learned vector; the capped feed-forward gate (library ``branches``) ---------------------
+
+def add_scaled_normed(x: torch.Tensor, terms, weights, scale: torch.Tensor | None, norm_w: torch.Tensor | None, eps: float,
+                      out_dtype: torch.dtype | None = None, rows: torch.Tensor | None = None):
+    """x += scale * sum_i weights[i] * terms[i] (one or two terms [n, width] of one element type; scale float32 [width] or
+    None; the sum in 32-bit, x float32 in place), and what the norm with weight ``norm_w`` makes of the sum, in
+    ``out_dtype``.  With ``rows`` only those rows are summed and normed and x stays as it is.  ``norm_w`` None: the sum
+    alone is made, and nothing is returned."""
+    _need(1 <= len(terms) <= 2 and len(weights) == len(terms), f"add_scaled_normed: {len(terms)} terms with {len(weights)} weights (one or two)")
+    _dev("add_scaled_normed", x, *terms, scale, norm_w, rows)
+    _i32("add_scaled_normed", rows)
+    n, width = x.shape
+    _need(x.dtype == F32 and all(t.shape == x.shape and t.dtype == terms[0].dtype for t in terms),
+          f"add_scaled_normed: x {tuple(x.shape)} {x.dtype}, terms {[tuple(t.shape) for t in terms]}")
+    for v in (scale, norm_w):
+        _need(v is None or (v.shape == (width,) and v.dtype == F32), f"add_scaled_normed: vectors are float32 [{width}]")
+    _need(norm_w is not None or rows is None, "add_scaled_normed: a selection of rows is for the norm that reads them")
+    n_out = n if rows is None else rows.shape[0]
+    out = torch.empty((n_out, width), dtype=out_dtype or F32, device=x.device) if norm_w is not None else None
+    library.call(branches(), "palm_add_scaled_normed", _stream(), _p(x), _p(terms[0]), float(weights[0]),
+                 _p(terms[1]) if len(terms) > 1 else None, float(weights[1]) if len(terms) > 1 else 0.0, _code(terms[0], "add_scaled_normed"),
+                 _p(scale), _p(norm_w), float(eps), _p(rows), n_out, width, int(rows is None), _p(out),
+                 _code(out, "add_scaled_normed out") if out is not None else 0)
+    return out
+
+
+def capped_gate(gate_up: torch.Tensor, limit: float, slope: float, shift: float) -> torch.Tensor:
+    """[n, 2 ff] (gate | up) -> [n, ff]: g * sigmoid(slope * g) * (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    _dev("capped_gate", gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, f"capped_gate: rows {tuple(gate_up.shape)} are not [n, 2 ff]")
+    n, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((n, ff), dtype=gate_up.dtype, device=gate_up.device)
+    library.call(branches(), "palm_capped_gate", _stream(), _p(gate_up), _p(out), _code(gate_up, "capped_gate"), n, ff, float(limit),
+                 float(slope), float(shift))
+    return out

@@ -2,8 +2,8 @@
 blocks, and the embedding and head at the two ends."""
 from .base import (CATEGORIES, Builder, StepContext, cache_needs, context_ints, make_context, part_class, register_part)
 from . import (norm, position, attention, feedforward, block, embedding, retention, selective_scan,  # noqa: F401  (registers the kinds)
-               differential_attention, delta_rule, latent_attention)
+               differential_attention, delta_rule, latent_attention, sink_attention, parallel)
 from .linear import Linear
-from .residual import Prenormed, ResidualSink, as_tensor, run_branch
+from .residual import Prenormed, ResidualSink, WeightedSum, as_tensor, run_branch
 
 __all__ = ["CATEGORIES", "Builder", "StepContext", "cache_needs", "context_ints", "make_context", "part_class", "register_part", "Linear"]

@@ -16,13 +16,18 @@ the rounded copy for the next reader are one kernel.
 ``sandwich``: x += gain * norm_b(mixer(norm_a(x))); x += gain * norm_d(feed_forward(norm_c(x))): a norm on each side of
 every branch and one multiplier on what is added.  A layer may have no feed-forward.  The norm of a branch's output, the
 scaled add and the norm that reads the stream next are one kernel.
+
+``pre_norm_scaled``: x += s1 * mixer(norm(x)); x += s2 * feed_forward(norm(x)) with learned vectors s1, s2 over the width
+("layer scale").  A layer may have no feed-forward.  A branch may hand back a sum that is still to be made (the sides of
+parallel mixers with their weights); the terms, the vector, the 32-bit add and the norm that reads the stream next are
+one kernel.
 """
 from __future__ import annotations
 
 from ..kernels import ops
 from .base import cache_needs, register_part
 from .norm import PassThrough
-from .residual import ResidualSink, as_tensor, run_branch
+from .residual import ResidualSink, WeightedSum, as_tensor, run_branch
 
 
 @register_part("block", "pre_norm")
@@ -140,3 +145,54 @@ class SandwichBlock:
         h = self._add(x, y, self.mixer_out_norm, self.feed_forward_norm, None)
         y = self.feed_forward.forward(h, ctx)
         return self._add(x, y, self.feed_forward_out_norm, sink.norm, sink.rows)
+
+
+@register_part("block", "pre_norm_scaled")
+class ScaledPreNormBlock:
+    def __init__(self, spec, builder):
+        self.mixer_norm = builder.build(spec.parts["mixer_norm"])
+        self.mixer = builder.build(spec.parts["mixer"])
+        self.mixer_scale = builder.tensor(spec, "mixer_scale") if "mixer_scale" in spec.tensors else None
+        self.feed_forward = builder.build(spec.parts["feed_forward"]) if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"]) if self.feed_forward is not None else None
+        self.feed_forward_scale = builder.tensor(spec, "feed_forward_scale") if "feed_forward_scale" in spec.tensors else None
+        self.dtype = builder.dtype
+        width = int(spec.params["hidden_size"])
+        for v in (self.mixer_scale, self.feed_forward_scale):
+            if v is not None and v.shape != (width,):
+                raise ValueError(f"a branch's scale is a vector over the width {width}, not {tuple(v.shape)}")
+
+    @property
+    def capturable(self) -> bool:
+        parts = [self.mixer_norm, self.mixer] + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
+        return all(getattr(p, "capturable", False) for p in parts)
+
+    @staticmethod
+    def cache_needs(spec):
+        return cache_needs(spec.parts["mixer"])
+
+    @property
+    def entry_norm(self):
+        return self.mixer_norm
+
+    def _add(self, x, y, scale, reader, rows):
+        """x += scale * y; returns what ``reader`` (the norm that reads x next) makes of x, over ``rows``."""
+        terms, weights = (y.terms, y.weights) if isinstance(y, WeightedSum) else ([y], [1.0])
+        while len(terms) > 2:                                   # the kernel adds two terms a pass
+            ops.add_scaled_normed(x, terms[:2], weights[:2], scale, None, 0.0)
+            terms, weights = terms[2:], weights[2:]
+        if getattr(reader, "folds_into_products", False):
+            if rows is not None:
+                # the rows that are read next: their sums are made for the norm alone; the stream is not needed again
+                return ops.add_scaled_normed(x, terms, weights, scale, reader.weight, reader.eps, self.dtype, rows=rows)
+            return ops.add_scaled_normed(x, terms, weights, scale, reader.weight, reader.eps, self.dtype)
+        ops.add_scaled_normed(x, terms, weights, scale, None, 0.0)
+        return reader(x, rows=rows)
+
+    def forward(self, x, h, ctx, sink):
+        y = self.mixer.forward(as_tensor(h), ctx)
+        if self.feed_forward is None:
+            return self._add(x, y, self.mixer_scale, sink.norm, sink.rows)
+        h = self._add(x, y, self.mixer_scale, self.feed_forward_norm, None)
+        y = self.feed_forward.forward(h, ctx)
+        return self._add(x, y, self.feed_forward_scale, sink.norm, sink.rows)

@@ -11,6 +11,9 @@ choice) pairs are grouped by expert on the device and all experts' rows go throu
 cores (bfloat16); in the float32 mode, and for sizes those do not take, the host groups the pairs and every expert's
 rows go through its two products as ``Linear`` makes them.
 
+``capped_gated``: down( g * sigmoid(slope * g) * (u + shift) ) with g = min(gate(h), limit) and u = clamp(up(h), -limit,
+limit); gate and up joined into one [2I, H] product.
+
 ``dense``: down(act(up(h))) with an activation chosen by name.  ``xielu`` has two learned numbers p, q (tensor
 ``activation``, float32 [2]): for z > 0, softplus(p) z^2 + z/2; for z <= 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
 from __future__ import annotations
@@ -42,6 +45,26 @@ class GatedSiluFeedForward:
 
     def forward(self, h, ctx, sink=None):
         return self.down(self.gate_up.gated(h), sink=sink)
+
+
+@register_part("feed_forward", "capped_gated")
+class CappedGatedFeedForward:
+    capturable = True
+
+    def __init__(self, spec, builder):
+        p = spec.params
+        self.hidden, self.inter = int(p["hidden_size"]), int(p["intermediate_size"])
+        self.limit, self.slope, self.shift = float(p["limit"]), float(p.get("slope", 1.0)), float(p.get("shift", 0.0))
+        if not self.limit > 0:
+            raise ValueError(f"feed-forward: limit = {self.limit} must be positive")
+        self.gate_up = Linear(builder.tensor(spec, "gate_up"))
+        self.down = Linear(builder.tensor(spec, "down"))
+        if self.gate_up.weight.shape != (2 * self.inter, self.hidden) or self.down.weight.shape != (self.hidden, self.inter):
+            raise ValueError(f"feed-forward: weights {tuple(self.gate_up.weight.shape)}, {tuple(self.down.weight.shape)} "
+                             f"do not fit hidden {self.hidden}, intermediate {self.inter}")
+
+    def forward(self, h, ctx):
+        return self.down(ops.capped_gate(self.gate_up(as_tensor(h)), self.limit, self.slope, self.shift))
 
 
 @register_part("feed_forward", "dense")

@@ -1,6 +1,7 @@
 """RMSNorm: y = x * (1 / sqrt(mean(x^2) + eps)) * w, statistics in 32-bit (kernels/norm.cpp:13-31).
 The residual add that precedes a norm in a block is fused into the same pass
-(engine/cuda_ops.cu:140-170 has the same fusion)."""
+(engine/cuda_ops.cu:140-170 has the same fusion).  With ``offset`` c the checkpoint stores w - c (a weight kept around
+zero for c = 1): the sum is made once, in 32-bit, when the part is built."""
 from __future__ import annotations
 
 import torch
@@ -19,6 +20,9 @@ class RMSNorm:
         self.width = int(spec.params["width"])
         self.eps = float(spec.params["eps"])
         self.weight = builder.tensor(spec, "weight")
+        offset = float(spec.params.get("offset", 0.0))
+        if offset:
+            self.weight = self.weight + offset
         self.dtype = builder.dtype
         if self.weight.shape != (self.width,):
             raise ValueError(f"RMSNorm of width {self.width} got a weight of shape {tuple(self.weight.shape)}")

@@ -37,9 +37,23 @@ class Prenormed:
         return ops.scale_rows(self.values, self.ss, self.eps)
 
 
+@dataclass
+class WeightedSum:
+    """A branch output that is still a sum to be made: sum_i weights[i] * terms[i], every term [n, width].  A block that
+    adds its branches in a 32-bit pass of its own takes the terms as they are; anything else calls ``materialize()``."""
+    terms: list
+    weights: list
+
+    def materialize(self) -> torch.Tensor:
+        total = torch.zeros(self.terms[0].shape, dtype=torch.float32, device=self.terms[0].device)
+        for i in range(0, len(self.terms), 2):
+            ops.add_scaled_normed(total, self.terms[i:i + 2], self.weights[i:i + 2], None, None, 0.0)
+        return total
+
+
 def as_tensor(h) -> torch.Tensor:
     """The normed rows as a plain tensor, whatever form they came in."""
-    return h.materialize() if isinstance(h, Prenormed) else h
+    return h.materialize() if isinstance(h, (Prenormed, WeightedSum)) else h
 
 
 class ResidualSink:

@@ -8,6 +8,11 @@ q and k are rotated first if the part has a ``position`` (k is multiplied by ``k
 head's o_t is divided by its root mean square (``eps`` inside the root, no weight); the heads are joined, multiplied by
 silu of a gate projection and projected back.  One joined product makes q | k | v | gate.  S is float32 and is kept
 per sequence (``StateNeed``); rotated values and everything in the recurrence are 32-bit whatever the run's type.
+
+Options that make it other linear attentions of the same recurrence: ``input_activation`` "silu" puts q, k and v through
+silu first; ``norm`` "joined" norms a token's heads together instead of each alone, o / sqrt(mean over all heads' values
+of o^2 + eps) times the weight tensor ``norm`` (float32 [heads * value_dim]); ``gate_activation`` "sigmoid" gates with
+the sigmoid of the gate rows instead of their silu.
 """
 from __future__ import annotations
 
@@ -38,9 +43,22 @@ class Retention:
                              f"of key size {self.dk} and value size {self.dv} over hidden {self.hidden}")
         if self.out.weight.shape != (self.hidden, self.nh * self.dv):
             raise ValueError(f"retention: output weight {tuple(self.out.weight.shape)} does not fit")
+        self.input_silu = self._choice(p, "input_activation", (None, "silu")) == "silu"
+        self.joined = self._choice(p, "norm", ("head_unit", "joined"), "head_unit") == "joined"
+        self.gate_sigmoid = self._choice(p, "gate_activation", ("silu", "sigmoid"), "silu") == "sigmoid"
+        self.norm_weight = builder.tensor(spec, "norm") if self.joined else None
+        if self.gate_sigmoid and not self.joined:
+            raise ValueError("retention: the per-head unit norm comes with a silu gate")
         self.position = builder.build(spec.parts["position"]) if "position" in spec.parts else None
         if self.position is not None and (self.position.pairing != "half_split" or self.position.rotary_dim > self.dk):
             raise ValueError("retention: the rotation pairs dimension i with i + rotary_dim/2 within the key size")
+
+    @staticmethod
+    def _choice(p, key, allowed, default=None):
+        value = p.get(key, default)
+        if value not in allowed:
+            raise ValueError(f"retention: {key} = {value!r} is not one of {allowed}")
+        return value
 
     @staticmethod
     def cache_needs(spec):
@@ -55,5 +73,6 @@ class Retention:
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         o = ops.retention(rows, self.nh, self.dk, self.dv, self.decay, self.key_scale, self.eps, lc.states["retention"], ctx,
-                          cos=cos, sin=sin, rot=self.position.rotary_dim if tables is not None else 0)
+                          cos=cos, sin=sin, rot=self.position.rotary_dim if tables is not None else 0,
+                          input_silu=self.input_silu, joined_norm=self.norm_weight, gate_sigmoid=self.gate_sigmoid)
         return self.out(o)
