@@ -22,10 +22,6 @@ def norm_around_one(x, w, eps):
     return unit_rows(x, eps) * (1.0 + w)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def rotation_frequencies(rot):
     """Pair i's angle per position, and the factor on cos and sin."""
     dims, base = int(rot["dims"]), float(rot["base"])
@@ -57,6 +53,36 @@ def rotate(x, positions, rot):
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], dim=-1)
 
 
+def sink_softmax_heads(q, k, v, positions, scale, size, sink=0.0):
+    """q [T, H, d], k [T, G, d], v [T, G, dv] of one sequence -> [T, H, dv].  A query at position i sees the keys j with
+    0 <= i - j < size (size None: every j <= i); the denominator has one more term, exp(sink), that carries no value
+    (sink None: an ordinary softmax)."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[-1], dtype=F64)
+    i, j = positions[:, None], positions[None, :]
+    seen = (i - j >= 0) if size is None else (i - j >= 0) & (i - j < size)
+    for hd in range(H):
+        g = hd // (H // G)
+        s = (q[:, hd] @ k[:, g].T) * scale
+        e = torch.where(seen, torch.exp(s), torch.zeros_like(s))
+        extra = 0.0 if sink is None else math.exp(sink)
+        out[:, hd] = (e / (extra + e.sum(-1, keepdim=True))) @ v[:, g]
+    return out
+
+
+def decay_recurrence(q, k, v, decay, state=None):
+    """q, k [T, H, d], v [T, H, dv]: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t.  Returns (o [T, H, dv], S)."""
+    T, H, d = q.shape
+    S = torch.zeros(H, d, v.shape[-1], dtype=F64) if state is None else state.clone()
+    o = torch.zeros(T, H, v.shape[-1], dtype=F64)
+    for t in range(T):
+        for hd in range(H):
+            S[hd] = float(decay[hd]) * S[hd] + torch.outer(k[t, hd], v[t, hd])
+            o[t, hd] = S[hd].T @ q[t, hd]
+    return o, S
+
+
 def window_sink_attention(h, w, m, eps, positions):
     """The left side.  h [T, width]; w: the side's tensors by short name ('q', 'q.b', 'q.norm', ..); m: its sizes."""
     T = h.shape[0]
@@ -70,15 +96,7 @@ def window_sink_attention(h, w, m, eps, positions):
     if m.get("rot"):
         q, k = rotate(q, positions, m["rot"]), rotate(k, positions, m["rot"])
     size = int(m["mask"]["size"]) if m.get("mask") else None
-    out = torch.zeros(T, H, dv, dtype=F64)
-    for hd in range(H):
-        g = hd // (H // G)
-        s = (q[:, hd] @ k[:, g].T) * float(m["scale"])                       # [T, T]
-        i, j = positions[:, None], positions[None, :]
-        seen = (i - j >= 0) if size is None else (i - j >= 0) & (i - j < size)
-        e = torch.where(seen, torch.exp(s), torch.zeros_like(s))
-        p = e / (1.0 + e.sum(-1, keepdim=True))                             # the one: a sink of score 0 without a value
-        out[:, hd] = p @ v[:, g]
+    out = sink_softmax_heads(q, k, v, positions, float(m["scale"]), size)
     gate = torch.sigmoid(h @ w["g"].T)
     return (out.reshape(T, H * dv) * gate) @ w["o"].T
 
@@ -91,13 +109,7 @@ def lightning_attention(h, w, m, eps, state=None):
     q = silu(h @ w["q"].T).reshape(T, H, d)
     k = silu(h @ w["k"].T).reshape(T, H, d)
     v = silu(h @ w["v"].T).reshape(T, H, dv)
-    decay = [float(x) for x in m["decay"]]
-    S = torch.zeros(H, d, dv, dtype=F64) if state is None else state.clone()
-    o = torch.zeros(T, H, dv, dtype=F64)
-    for t in range(T):
-        for hd in range(H):
-            S[hd] = decay[hd] * S[hd] + torch.outer(k[t, hd], v[t, hd])
-            o[t, hd] = S[hd].T @ q[t, hd]
+    o, S = decay_recurrence(q, k, v, m["decay"], state)
     o = unit_rows(o.reshape(T, H * dv), eps) * w["norm"]                     # all heads normed together
     return (o * torch.sigmoid(h @ w["g"].T)) @ w["o"].T, S
 
@@ -160,3 +172,19 @@ def forward(cfg, tensors, tokens, layers_out=None):
             layers_out.append(x.clone())
     x = norm_around_one(x, tensors["final.norm"].to(F64), float(cfg["norm"]["eps"]))
     return x @ table.T
+
+
+def read_model(path):
+    """(raw config, tensors by name) of a model folder."""
+    import json
+    from pathlib import Path
+    from safetensors.torch import load_file
+    path = Path(path)
+    return json.loads((path / "config.json").read_text()), load_file(str(path / "model.safetensors"))
+
+
+def greedy(cfg, tensors, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(cfg, tensors, ids)[-1].argmax()))
+    return ids[len(prompt):]
