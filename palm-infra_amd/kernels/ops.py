@@ -1521,8 +1521,55 @@ def sink_attention_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, he
     return out
 
 
+_SINK_MFMA_SIGNATURE = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_int, c_void_p]
+_sink_mfma_libs: dict = {}
+
+
+def sink_mfma_serves(q: torch.Tensor, dim: int, vdim: int) -> bool:
+    """Whether the matrix-core kernel takes these queries: bfloat16, a key size in steps of 8 and a value size in steps of 4."""
+    return q.dtype == BF16 and dim % 8 == 0 and vdim % 4 == 0 and dim <= 256 and vdim <= 256
+
+
+def sink_attention_mfma_lib(dim: int, vdim: int):
+    """The library compiled for this key and value size (built when a model of these sizes first runs a prompt)."""
+    key = (-(-dim // 32), -(-vdim // 16))
+    lib = _sink_mfma_libs.get(key)
+    if lib is None:
+        lib = library.load(f"sink_attention_k{key[0]}_v{key[1]}")
+        lib.palm_sink_attention_mfma.argtypes, lib.palm_sink_attention_mfma.restype = _SINK_MFMA_SIGNATURE, c_int
+        _sink_mfma_libs[key] = lib
+    return lib
+
+
+def sink_attention_mfma(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
+                        scale: float, window: int | None, sink: float | None, gate: torch.Tensor | None, gate_off: int = 0) -> torch.Tensor:
+    """``sink_attention_exact`` for prompts in bfloat16 on the matrix cores (scores, weights and sums 32-bit)."""
+    _dev("sink_attention_mfma", q, k_cache, v_cache, block_table, gate, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _i32("sink_attention_mfma", block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    n = q.shape[0]
+    _need(sink_mfma_serves(q, dim, vdim), f"sink_attention_mfma: {q.dtype} queries of key size {dim} and value size {vdim} are not served")
+    _need(q.shape == (ctx.n_tokens, heads, dim), f"sink_attention_mfma: q {tuple(q.shape)} is not [{ctx.n_tokens}, {heads}, {dim}]")
+    _need(k_cache.dtype == BF16 and v_cache.dtype == BF16 and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
+          and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS), f"sink_attention_mfma: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= gate_off + heads * vdim and gate.dtype == BF16,
+              f"sink_attention_mfma: gate rows {tuple(gate.shape)} {gate.dtype} from column {gate_off}")
+        gate_ptr, gate_stride = gate.data_ptr() + gate_off * gate.element_size(), gate.shape[1]
+    out = torch.empty((n, heads * vdim), dtype=BF16, device=q.device)
+    library.call(sink_attention_mfma_lib(dim, vdim), "palm_sink_attention_mfma", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
+                 heads, kv_heads, dim, vdim, float(scale), int(window or 0), int(sink is not None), float(sink or 0.0), gate_ptr,
+                 gate_stride, _p(out))
+    return out
+
+
 def sink_attention(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off=0):
-    """The kernel that serves: the exact one for the float32 mode and for single tokens."""
+    """The kernel that serves: the matrix cores for prompts in bfloat16, the exact one for the float32 mode, for single
+    tokens, and for sizes that the matrix-core kernel does not take."""
+    if not ctx.is_decode and sink_mfma_serves(q, dim, vdim):
+        return sink_attention_mfma(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off)
     return sink_attention_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off)
 
 

@@ -343,23 +343,28 @@ def test_q_k_v_pass_bias_norms_part_rotation_and_pages(dtype, norm):
     assert float(kc[-1].abs().max()) == 0.0 and float(vc[-1].abs().max()) == 0.0        # the page that pads is not written
 
 
-def _attend(dtype, H, G, d, dv, window, sink, q, k, v, gate, prompt_cut, slices):
-    """q, k, v of one sequence through the kernels: the first ``prompt_cut`` tokens in one step, the others one a step (with
-    ``slices`` slices of their key range); returns [T, H * dv]."""
+def _attend(dtype, H, G, d, dv, window, sink, q, k, v, gate, prompt_cut, slices, exact=True):
+    """q, k, v of one sequence through the kernels: the first ``prompt_cut`` tokens in one step (or, a list: in steps of these
+    sizes), the others one a step (with ``slices`` slices of their key range); returns [T, H * dv].  ``exact`` False: the
+    kernel that the parts would get (the matrix cores for portions in bfloat16)."""
     from palm_infra_amd.kernels import ops
     T = q.shape[0]
     kc, vc, table = _paged(1, -(-T // 64) + 1, G, d, dv, TORCH[dtype], seed=T)
     outs = []
     at = 0
-    for count in [prompt_cut] + [1] * (T - prompt_cut):
+    cuts = list(prompt_cut) if isinstance(prompt_cut, (list, tuple)) else [prompt_cut]
+    for count in cuts + [1] * (T - sum(cuts)):
         if count == 0:
             continue
         ctx = _step_context([at], [count])
         rows = torch.cat([q[at:at + count].reshape(count, -1), k[at:at + count].reshape(count, -1), v[at:at + count].reshape(count, -1),
                           gate[at:at + count]], dim=1).to(TORCH[dtype]).cuda()
         qq = ops.sink_qkv_store(rows, H, G, d, dv, None, None, None, None, 0.0, None, None, 0, kc, vc, table, ctx)
-        outs.append(ops.sink_attention_exact(qq, kc, vc, table, ctx, H, G, d, dv, 0.3, window, sink, rows, H * d + G * d + G * dv,
-                                             slices=1 if count > 1 else slices))
+        if exact:
+            outs.append(ops.sink_attention_exact(qq, kc, vc, table, ctx, H, G, d, dv, 0.3, window, sink, rows, H * d + G * d + G * dv,
+                                                 slices=1 if count > 1 else slices))
+        else:
+            outs.append(ops.sink_attention(qq, kc, vc, table, ctx, H, G, d, dv, 0.3, window, sink, rows, H * d + G * d + G * dv))
         at += count
     return torch.cat(outs).cpu().double()
 
@@ -406,6 +411,15 @@ def test_attention_kernel_far_keys_page_borders_window_edges_and_the_sink(dtype,
         assert torch.allclose(got, want, **tol), (cut, slices, float((got - want).abs().max()), int((got - want).abs().max(-1).values.argmax()))
     no_sink = _attend(dtype, H, G, d, dv, window, None, q, k, v, gate, T - 3, 2)
     assert torch.allclose(no_sink, plain, **tol)
+    if dtype == "bfloat16":
+        # the kernels that the parts get: the matrix cores for the portions (the weights are rounded to bfloat16 there)
+        from palm_infra_amd.kernels import ops
+        assert ops.sink_mfma_serves(torch.empty(0, dtype=torch.bfloat16), d, dv) == (d % 8 == 0 and dv % 4 == 0)
+        for cuts in (T, [T - 2], [50, 33, 17, 98], [2, 3, 64, 65, 7], [129, 70]):
+            got = _attend(dtype, H, G, d, dv, window, 0.0, q, k, v, gate, cuts, 1, exact=False)
+            assert torch.allclose(got, want, atol=0.03, rtol=0.03), (cuts, float((got - want).abs().max()), int((got - want).abs().max(-1).values.argmax()))
+        no_sink = _attend(dtype, H, G, d, dv, window, None, q, k, v, gate, [T - 30, 20], 1, exact=False)
+        assert torch.allclose(no_sink, plain, atol=0.03, rtol=0.03)
 
 
 @gpu
