@@ -362,6 +362,14 @@ def _mixer_rooflines(raw: dict, tokens: int, batch: int, context: int) -> dict:
                 out["palm_latent_attention"] = (flops, mfma, 2.0 * batch * min(context, w) * row, hbm)
                 # the prompt kernel also applies the value matrices
                 out["palm_latent_attention_mfma"] = (flops + 2.0 * tokens * m["heads"] * m["kv_rank"] * m["vdim"], mfma, None, None)
+            elif layer["type"] == "parallel" and "palm_sink_attention" not in out:
+                a, r = m["left"], m["right"]
+                w = a["mask"]["size"] if a.get("mask") else tokens
+                seen = sum(min(p + 1, w) for p in range(tokens))
+                out["palm_sink_attention_mfma"] = (2.0 * a["heads"] * (a["dim"] + a["vdim"]) * seen, mfma, None, None)
+                out["palm_sink_attention"] = (None, None, 2.0 * batch * min(context, w) * a["kv_heads"] * (a["dim"] + a["vdim"]), hbm)
+                per = r["heads"] * r["dim"] * r["vdim"]
+                out["palm_retention"] = (4.0 * tokens * per, vec, 2.0 * 4 * batch * per, hbm)
             if layer.get("mlp") and layer["mlp"].get("kind") == "moe" and "palm_moe_experts" not in out:
                 f = layer["mlp"]
                 out["palm_moe_experts"] = (None, None, 2.0 * batch * f["router"]["top"] * 3 * f["expert"]["ff"] * raw["width"], hbm)
@@ -443,7 +451,18 @@ def _pazilorn_bench(args, record) -> dict:
     return record["sizes"]["pazilorn-2048"]["pazilorn"]
 
 
-DESIGNS = {"sebesun": ("Sebesun presets beside Qwen3 models of equal width and depth", _sebesun_bench),
+def _matalix_bench(args, record) -> dict:
+    """The Matalix presets beside the Sebesun presets of the same width and depth (the closest design here: the same
+    recurrence with one decay per head, and attention with a value size of its own on the matrix cores)."""
+    for width in ("2048", "4096"):
+        record["sizes"][f"matalix-{width}"] = {
+            "matalix": design_points(preset_dict(f"matalix-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT),
+            "sebesun": design_points(preset_dict(f"sebesun-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT)}
+    return record["sizes"]["matalix-2048"]["matalix"]
+
+
+DESIGNS = {"matalix": ("Matalix presets beside Sebesun presets of equal width and depth", _matalix_bench),
+           "sebesun": ("Sebesun presets beside Qwen3 models of equal width and depth", _sebesun_bench),
            "pazilorn": ("Pazilorn presets beside Sebesun presets of equal width and depth", _pazilorn_bench)}
 
 
@@ -479,7 +498,7 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="tokens of the timed prompt (2,048 is the workload's; others serve profiles of longer prompts)")
     ap.add_argument("--design", help="instead of the default workload: another design's presets beside its closest relative "
-                    "of equal width and depth ('sebesun' beside Qwen3, 'pazilorn' beside Sebesun)")
+                    "of equal width and depth ('sebesun' beside Qwen3, 'pazilorn' and 'matalix' beside Sebesun)")
     args = ap.parse_args(argv)
     if args.design:
         if args.gpus != 1:

@@ -102,8 +102,8 @@ class MatalixConfig:
         out = {k: _positive(_get(m, k, int, where), f"{where}.{k}") for k in ("heads", "kv_heads", "dim", "vdim")}
         if out["heads"] % out["kv_heads"]:
             raise ConfigError(f"config.json: {where}: {out['heads']} heads are not a multiple of {out['kv_heads']} kv heads")
-        if out["dim"] > 512 or out["vdim"] > 512:
-            raise ConfigError(f"config.json: {where}: the attention kernels take key and value sizes up to 512")
+        if out["dim"] > 256 or out["vdim"] > 256:
+            raise ConfigError(f"config.json: {where}: the attention kernels take key and value sizes up to 256")
         out["scale"] = _get(m, "scale", float, where)
         mask = m.get("mask")
         out["mask"] = {"size": _positive(_get(mask, "size", int, where + ".mask"), where + ".mask.size")} if mask else None
@@ -162,24 +162,30 @@ class MatalixConfig:
             "mixer", "sink_attention",
             {"hidden_size": W, "num_heads": H, "num_kv_heads": G, "key_dim": d, "value_dim": dv, "scale": m["scale"],
              "window": m["mask"]["size"] if m["mask"] else None, "eps": self.eps, "qk_norm": "projection", "sink": True,
-             "gate": "sigmoid"},
-            {"qkvg": joined((p + "q", p + "k", p + "v", p + "g"), ((H * d, W), (G * d, W), (G * dv, W), (H * dv, W)), "matrix",
-                            ("normal", 0.0, 0.1)),
-             "qkv_bias": joined((p + "q.b", p + "k.b", p + "v.b"), ((H * d,), (G * d,), (G * dv,)), "vector", ("normal", 0.0, 0.3)),
+             "gate": "sigmoid", "input": "shared"},
+            {"qkv_bias": joined((p + "q.b", p + "k.b", p + "v.b"), ((H * d,), (G * d,), (G * dv,)), "vector", ("normal", 0.0, 0.3)),
              "q_norm": tensor(p + "q.norm", (H * d,), "vector", ("normal", 1.2, 0.4)),
              "k_norm": tensor(p + "k.norm", (G * d,), "vector", ("normal", 1.2, 0.4)),
              "out": tensor(p + "o", (W, H * dv), "matrix", ("normal", 0.0, 0.06))},
             parts)
+
+    def _shared_input(self, p: str, m: dict):
+        """Both sides' input matrices as one: left q | k | v | g, then right q | k | v | g (one product a layer reads the
+        normed rows once)."""
+        W, a, r = self.width, m["left"], m["right"]
+        H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+        names = [p + "left." + n for n in "qkvg"] + [p + "right." + n for n in "qkvg"]
+        shapes = [(H * d, W), (G * d, W), (G * dv, W), (H * dv, W),
+                  (r["heads"] * r["dim"], W), (r["heads"] * r["dim"], W), (r["heads"] * r["vdim"], W), (r["heads"] * r["vdim"], W)]
+        return joined(names, shapes, "matrix", ("normal", 0.0, 0.1))
 
     def _right(self, p: str, m: dict) -> PartSpec:
         W, H, d, dv = self.width, m["heads"], m["dim"], m["vdim"]
         return PartSpec(
             "mixer", "retention",
             {"hidden_size": W, "num_heads": H, "key_dim": d, "value_dim": dv, "decay": tuple(m["decay"]), "key_scale": 1.0,
-             "eps": self.eps, "input_activation": "silu", "norm": "joined", "gate_activation": "sigmoid"},
-            {"qkvg": joined((p + "q", p + "k", p + "v", p + "g"), ((H * d, W), (H * d, W), (H * dv, W), (H * dv, W)), "matrix",
-                            ("normal", 0.0, 0.1)),
-             "norm": tensor(p + "norm", (H * dv,), "vector", _AROUND_ONE),
+             "eps": self.eps, "input_activation": "silu", "norm": "joined", "gate_activation": "sigmoid", "input": "shared"},
+            {"norm": tensor(p + "norm", (H * dv,), "vector", _AROUND_ONE),
              "out": tensor(p + "o", (W, H * dv), "matrix", ("normal", 0.0, 0.1))})
 
     def spec(self, tensor_names=None) -> ModelSpec:
@@ -193,7 +199,8 @@ class MatalixConfig:
         for i, layer in enumerate(self.layers):
             p, m = f"l{i}.", layer["mixer"]
             parts = {"mixer_norm": norm(p + "norm1"),
-                     "mixer": PartSpec("mixer", "parallel", {"weights": (m["left_scale"], m["right_scale"])}, {},
+                     "mixer": PartSpec("mixer", "parallel", {"weights": (m["left_scale"], m["right_scale"])},
+                                       {"in": self._shared_input(p + "mix.", m)},
                                        {"left": self._left(p + "mix.left.", m["left"]), "right": self._right(p + "mix.right.", m["right"])})}
             scales = {"mixer_scale": tensor(p + "ls1", (W,), "vector", ("normal", 0.8, 0.2))}
             f = layer["mlp"]

@@ -30,7 +30,7 @@ enum SinkNorm : int { SK_NORM_NONE = 0, SK_NORM_PROJECTION = 1, SK_NORM_HEAD = 2
 // One block per token.  The projection-wide sums of squares are made by the whole block; then a wave takes a head
 // (of q or of k) at a time: norm, weight, rotation, and q goes to q_out, k to its page.
 template <typename T>
-__global__ __launch_bounds__(256) void sink_qkv_store_kernel(
+__global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
     const T* __restrict__ rows, int stride, int q_off, int k_off, int v_off, const float* __restrict__ bias,
     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ tok_slot, const int* __restrict__ positions, int norm_mode, const float* __restrict__ q_w,
@@ -109,8 +109,10 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "sink_qkv_store: a rotation needs its cos and sin rows");
     PALM_CHECK(!write_cache || (k_cache && v_cache && block_table && tok_slot && max_pages > 0), "sink_qkv_store: writing needs cache, pages and slots");
     if (n_tokens == 0) return 0;
+    // a wave takes a head at a time: as many waves as there are heads of q and k, within a block's sixteen
+    const int threads = min(1024, max(256, WAVE * (heads + kv_heads)));
     PALM_DTYPE_SWITCH(dtype, T,
-        sink_qkv_store_kernel<T><<<n_tokens, 256, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
+        sink_qkv_store_kernel<T><<<n_tokens, threads, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
                                                               (T*)v_cache, block_table, max_pages, tok_slot, positions, norm_mode, q_w, k_w,
                                                               eps, cos_t, sin_t, rot, heads, kv_heads, dim, vdim, write_cache));
     PALM_LAUNCHED();

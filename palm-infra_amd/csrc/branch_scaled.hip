@@ -11,7 +11,7 @@
 // One block per row that is read next (`rows` selects them; without a selection every row, and x is updated).  The
 // row's sums wait in LDS between the pass that makes them and the pass that norms them.
 template <typename TD, typename TO>
-__global__ __launch_bounds__(256) void add_scaled_normed_kernel(float* __restrict__ x, const TD* __restrict__ d0, float c0,
+__global__ __launch_bounds__(1024) void add_scaled_normed_kernel(float* __restrict__ x, const TD* __restrict__ d0, float c0,
                                                                 const TD* __restrict__ d1, float c1, const float* __restrict__ ls,
                                                                 const float* __restrict__ w, float eps, const int* __restrict__ rows,
                                                                 int width, int update, TO* __restrict__ out) {
@@ -44,9 +44,10 @@ PALM_API int palm_add_scaled_normed(hipStream_t stream, float* x, const void* d0
     PALM_CHECK(!(rows && update), "add_scaled_normed: a selection of rows leaves the stream as it is");
     PALM_CHECK(rows || update, "add_scaled_normed: without a selection of rows the stream is updated");
     const size_t lds = (size_t)width * sizeof(float);
+    const int threads = width >= 2048 ? 1024 : width >= 1024 ? 512 : 256;      // a wide row has two values a thread: short chains of loads
     PALM_DTYPE_SWITCH(d_dtype, TD, {
         PALM_DTYPE_SWITCH(out_dtype, TO,
-            add_scaled_normed_kernel<TD, TO><<<n_out, 256, lds, stream>>>(x, (const TD*)d0, c0, (const TD*)d1, c1, ls, w, eps, rows, width,
+            add_scaled_normed_kernel<TD, TO><<<n_out, threads, lds, stream>>>(x, (const TD*)d0, c0, (const TD*)d1, c1, ls, w, eps, rows, width,
                                                                          update, (TO*)out));
     });
     PALM_LAUNCHED();

@@ -250,7 +250,7 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
 // heads), f = sigmoid (gate_act 1) or silu (gate_act 0).  raw is 32-bit; the gate lies in rows `gate_stride` elements
 // apart.  One block per token.
 template <typename T>
-__global__ __launch_bounds__(256) void joined_norm_gate_kernel(const float* __restrict__ raw, const float* __restrict__ weight, float eps,
+__global__ __launch_bounds__(1024) void joined_norm_gate_kernel(const float* __restrict__ raw, const float* __restrict__ weight, float eps,
                                                                const T* __restrict__ gate, int gate_stride, int gate_act, int width,
                                                                T* __restrict__ out) {
     __shared__ float scratch[16];
@@ -272,7 +272,7 @@ PALM_API int palm_joined_norm_gate(hipStream_t stream, const float* raw, const f
     PALM_CHECK(gate_act == 0 || gate_act == 1, "joined_norm_gate: gate activation %d is neither silu (0) nor sigmoid (1)", gate_act);
     if (n_tokens == 0) return 0;
     PALM_DTYPE_SWITCH(dtype, T,
-        joined_norm_gate_kernel<T><<<n_tokens, 256, 0, stream>>>(raw, weight, eps, (const T*)gate, gate_stride, gate_act, width, (T*)out));
+        joined_norm_gate_kernel<T><<<n_tokens, width >= 2048 ? 1024 : width >= 1024 ? 512 : 256, 0, stream>>>(raw, weight, eps, (const T*)gate, gate_stride, gate_act, width, (T*)out));
     PALM_LAUNCHED();
     return 0;
 }

@@ -909,19 +909,20 @@ def retention_chunk(n_seqs: int, heads: int, max_new: int) -> int:
 
 def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, k_scale: float, eps: float,
               state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0, chunk: int | None = None, input_silu: bool = False,
-              joined_norm: torch.Tensor | None = None, gate_sigmoid: bool = False) -> torch.Tensor:
+              joined_norm: torch.Tensor | None = None, gate_sigmoid: bool = False, col0: int = 0) -> torch.Tensor:
     """The step's tokens through a retention layer's recurrence.  qkvg [n, heads * (2 dim + 2 vdim)] holds q | k | v |
     gate; state float32 [slots, heads, dim, vdim] is read and left updated.  Returns [n, heads * vdim]: the heads'
     outputs, unit-normed per head and gated by silu of the gate.  ``chunk``: see ``retention_chunk`` (None: chosen here).
 
     ``input_silu``: q, k and v go through silu first.  ``joined_norm`` (float32 [heads * vdim]): instead of the unit norm
     per head, a token's joined heads are normed together and multiplied by this weight; ``gate_sigmoid``: the gate is then
-    sigmoid of the gate values instead of silu."""
+    sigmoid of the gate values instead of silu.  ``col0``: q | k | v | gate begin at this column of wider rows (a product
+    that several mixers share)."""
     _dev("retention", qkvg, decay, state, cos, sin, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     _i32("retention", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     n = qkvg.shape[0]
-    _need(qkvg.dim() == 2 and qkvg.shape[1] == heads * (2 * dim + 2 * vdim), f"retention: rows {tuple(qkvg.shape)} are not "
-          f"[n, {heads} * (2*{dim} + 2*{vdim})]")
+    _need(qkvg.dim() == 2 and col0 >= 0 and qkvg.shape[1] >= col0 + heads * (2 * dim + 2 * vdim) and (col0 or qkvg.shape[1] == heads * (2 * dim + 2 * vdim)),
+          f"retention: rows {tuple(qkvg.shape)} from column {col0} are not [n, {heads} * (2*{dim} + 2*{vdim})]")
     _need(decay.shape == (heads,) and decay.dtype == F32, f"retention: one float32 decay for each of {heads} heads")
     _need(state.dim() == 4 and state.shape[1:] == (heads, dim, vdim) and state.dtype == F32,
           f"retention: state {tuple(state.shape)} {state.dtype} is not float32 [slots, {heads}, {dim}, {vdim}]")
@@ -944,9 +945,9 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
     if chunk:
         max_chunks = -(-ctx.max_new // chunk)
         starts = torch.empty((ctx.n_seqs * max_chunks, heads, dim, vdim), dtype=F32, device=qkvg.device)
-    g_off = 2 * heads * dim + heads * vdim
-    library.call(recurrent(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
-                 2 * heads * dim, g_off, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
+    g_off = col0 + 2 * heads * dim + heads * vdim
+    library.call(recurrent(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], col0, col0 + heads * dim,
+                 col0 + 2 * heads * dim, g_off, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
                  _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out),
                  int(ctx.max_new), chunk, _p(starts), n, _p(rotated), int(input_silu), int(raw is not None), _p(raw))
     if raw is not None:
@@ -1449,17 +1450,17 @@ SINK_BLOCKS_WANTED = 1024         # a decode step's key ranges are cut into slic
 
 
 def sink_qkv_store(rows: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, bias, norm: str | None, q_w, k_w, eps: float,
-                   cos, sin, rot: int, k_cache, v_cache, block_table, ctx, write_cache: bool = True) -> torch.Tensor:
+                   cos, sin, rot: int, k_cache, v_cache, block_table, ctx, write_cache: bool = True, col0: int = 0) -> torch.Tensor:
     """q, k and v of the step's tokens from ``rows`` [n, >= heads*dim + kv_heads*dim + kv_heads*vdim] (q | k | v | whatever
     follows): ``bias`` (float32 over q | k | v, or None) is added, q and k are normed (``norm``: "projection": one RMS norm
     over the whole q row and one over the whole k row, weights of those sizes; "head": per head, weights of the key size;
     None), their first ``rot`` dimensions are rotated by the tokens' cos and sin rows, k and v go to their pages, and q
-    comes back as [n, heads, dim]."""
+    comes back as [n, heads, dim].  ``col0``: q begins at this column of the rows."""
     _dev("sink_qkv_store", rows, bias, q_w, k_w, cos, sin, k_cache, v_cache, block_table, ctx.tok_slot, ctx.positions)
     _i32("sink_qkv_store", block_table, ctx.tok_slot, ctx.positions)
     n = rows.shape[0]
     q_size, k_size, v_size = heads * dim, kv_heads * dim, kv_heads * vdim
-    _need(rows.dim() == 2 and rows.shape[1] >= q_size + k_size + v_size and n == ctx.n_tokens,
+    _need(rows.dim() == 2 and col0 >= 0 and rows.shape[1] >= col0 + q_size + k_size + v_size and n == ctx.n_tokens,
           f"sink_qkv_store: rows {tuple(rows.shape)} for {ctx.n_tokens} tokens of {q_size} + {k_size} + {v_size}")
     _need(norm in SINK_NORMS, f"sink_qkv_store: norm {norm!r} is not one of {sorted(map(str, SINK_NORMS))}")
     if bias is not None:
@@ -1475,8 +1476,8 @@ def sink_qkv_store(rows: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim
           and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS) and block_table.dim() == 2,
           f"sink_qkv_store: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} for rows of {rows.dtype}")
     q = torch.empty((n, heads, dim), dtype=rows.dtype, device=rows.device)
-    library.call(sink_attention_lib(), "palm_sink_qkv_store", _stream(), _p(rows), _code(rows, "sink_qkv_store"), rows.shape[1], 0, q_size,
-                 q_size + k_size, _p(bias), _p(q), _p(k_cache), _p(v_cache), _p(block_table), block_table.shape[1], _p(ctx.tok_slot),
+    library.call(sink_attention_lib(), "palm_sink_qkv_store", _stream(), _p(rows), _code(rows, "sink_qkv_store"), rows.shape[1], col0, col0 + q_size,
+                 col0 + q_size + k_size, _p(bias), _p(q), _p(k_cache), _p(v_cache), _p(block_table), block_table.shape[1], _p(ctx.tok_slot),
                  _p(ctx.positions), SINK_NORMS[norm], _p(q_w), _p(k_w), float(eps), _p(cos), _p(sin), int(rot), n, heads, kv_heads, dim,
                  vdim, int(write_cache))
     return q

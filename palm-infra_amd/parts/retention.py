@@ -36,9 +36,12 @@ class Retention:
         if len(p["decay"]) != self.nh:
             raise ValueError(f"retention: {len(p['decay'])} decays for {self.nh} heads")
         self.decay = torch.tensor([float(d) for d in p["decay"]], dtype=torch.float32).to(builder.device)
-        self.qkvg = Linear(builder.tensor(spec, "qkvg"))
+        # the joined product is this part's own, or a wider one that the mixers beside it share (``input`` "shared")
+        self.shared_input = p.get("input") == "shared"
+        self.qkvg = None if self.shared_input else Linear(builder.tensor(spec, "qkvg"))
         self.out = Linear(builder.tensor(spec, "out"))
-        if self.qkvg.weight.shape != (self.nh * 2 * (self.dk + self.dv), self.hidden):
+        self.in_rows = self.nh * 2 * (self.dk + self.dv)
+        if self.qkvg is not None and self.qkvg.weight.shape != (self.in_rows, self.hidden):
             raise ValueError(f"retention: joined q/k/v/gate weight {tuple(self.qkvg.weight.shape)} does not fit {self.nh} heads "
                              f"of key size {self.dk} and value size {self.dv} over hidden {self.hidden}")
         if self.out.weight.shape != (self.hidden, self.nh * self.dv):
@@ -66,13 +69,18 @@ class Retention:
         return [StateNeed("retention", (int(p["num_heads"]), int(p["key_dim"]), int(p["value_dim"])))]
 
     def forward(self, h, ctx):
+        if self.qkvg is None:
+            raise RuntimeError("retention whose input product is shared gets its rows from the part that makes them")
+        return self.forward_rows(self.qkvg(h), 0, ctx)
+
+    def forward_rows(self, rows, col0, ctx):
+        """``rows`` [n, >= col0 + in_rows]: q | k | v | gate from column ``col0``."""
         lc = ctx.layer_cache
         if lc is None or not lc.states or "retention" not in lc.states:
             raise RuntimeError("retention needs its state; the step gave it no cache")
-        rows = self.qkvg(h)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         o = ops.retention(rows, self.nh, self.dk, self.dv, self.decay, self.key_scale, self.eps, lc.states["retention"], ctx,
                           cos=cos, sin=sin, rot=self.position.rotary_dim if tables is not None else 0,
-                          input_silu=self.input_silu, joined_norm=self.norm_weight, gate_sigmoid=self.gate_sigmoid)
+                          input_silu=self.input_silu, joined_norm=self.norm_weight, gate_sigmoid=self.gate_sigmoid, col0=col0)
         return self.out(o)

@@ -41,12 +41,14 @@ class SinkAttention:
             raise ValueError(f"sink attention: qk_norm {self.qk_norm!r} is one of {QK_NORMS}, gate {self.gate!r} one of {GATES}")
         if self.nh % self.nkv:
             raise ValueError(f"{self.nh} heads are not a multiple of {self.nkv} kv heads")
-        self.qkvg = Linear(builder.tensor(spec, "qkvg"))
+        # the joined product is this part's own, or a wider one that the mixers beside it share (``input`` "shared")
+        self.shared_input = p.get("input") == "shared"
+        self.qkvg = None if self.shared_input else Linear(builder.tensor(spec, "qkvg"))
         self.out = Linear(builder.tensor(spec, "out"))
         self.bias = builder.tensor(spec, "qkv_bias") if "qkv_bias" in spec.tensors else None
         self.gate_off = self.nh * self.dk + self.nkv * (self.dk + self.dv)
-        rows = self.gate_off + (self.nh * self.dv if self.gate else 0)
-        if self.qkvg.weight.shape != (rows, self.hidden):
+        self.in_rows = self.gate_off + (self.nh * self.dv if self.gate else 0)
+        if self.qkvg is not None and self.qkvg.weight.shape != (self.in_rows, self.hidden):
             raise ValueError(f"sink attention: joined weight {tuple(self.qkvg.weight.shape)} does not fit {self.nh} heads and {self.nkv} kv "
                              f"heads of key size {self.dk} and value size {self.dv} over hidden {self.hidden}")
         if self.out.weight.shape != (self.hidden, self.nh * self.dv):
@@ -65,16 +67,21 @@ class SinkAttention:
                        value_dim=int(p["value_dim"]))]
 
     def forward(self, h, ctx):
+        if self.qkvg is None:
+            raise RuntimeError("sink attention whose input product is shared gets its rows from the part that makes them")
+        return self.forward_rows(self.qkvg(h), 0, ctx)
+
+    def forward_rows(self, rows, col0, ctx):
+        """``rows`` [n, >= col0 + in_rows]: q | k | v (| gate) from column ``col0``."""
         lc = ctx.layer_cache
         if lc is None or lc.kv is None:
             raise RuntimeError("sink attention needs the keys and values of its layer; the step gave it no cache")
-        rows = self.qkvg(h)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         rot = self.position.rotary_dim if tables is not None else 0
         table = lc.kv.table_dev
         q = ops.sink_qkv_store(rows, self.nh, self.nkv, self.dk, self.dv, self.bias, self.qk_norm, self.q_w, self.k_w, self.eps,
-                               cos, sin, rot, lc.k, lc.v, table, ctx, write_cache=lc.writes)
+                               cos, sin, rot, lc.k, lc.v, table, ctx, write_cache=lc.writes, col0=col0)
         o = ops.sink_attention(q, lc.k, lc.v, table, ctx, self.nh, self.nkv, self.dk, self.dv, self.scale, self.window, self.sink,
-                               rows if self.gate else None, self.gate_off)
+                               rows if self.gate else None, col0 + self.gate_off)
         return self.out(o)
