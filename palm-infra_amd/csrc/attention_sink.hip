@@ -109,8 +109,9 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "sink_qkv_store: a rotation needs its cos and sin rows");
     PALM_CHECK(!write_cache || (k_cache && v_cache && block_table && tok_slot && max_pages > 0), "sink_qkv_store: writing needs cache, pages and slots");
     if (n_tokens == 0) return 0;
-    // a wave takes a head at a time: as many waves as there are heads of q and k, within a block's sixteen
-    const int threads = min(1024, max(256, WAVE * (heads + kv_heads)));
+    // a wave takes a head at a time: for few tokens (a decode step) as many waves as there are heads of q and k, within a
+    // block's sixteen; many tokens fill the chip anyway
+    const int threads = n_tokens >= 256 ? 256 : min(1024, max(256, WAVE * (heads + kv_heads)));
     PALM_DTYPE_SWITCH(dtype, T,
         sink_qkv_store_kernel<T><<<n_tokens, threads, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
                                                               (T*)v_cache, block_table, max_pages, tok_slot, positions, norm_mode, q_w, k_w,

@@ -44,7 +44,8 @@ PALM_API int palm_add_scaled_normed(hipStream_t stream, float* x, const void* d0
     PALM_CHECK(!(rows && update), "add_scaled_normed: a selection of rows leaves the stream as it is");
     PALM_CHECK(rows || update, "add_scaled_normed: without a selection of rows the stream is updated");
     const size_t lds = (size_t)width * sizeof(float);
-    const int threads = width >= 2048 ? 1024 : width >= 1024 ? 512 : 256;      // a wide row has two values a thread: short chains of loads
+    // few rows (a decode step): a wide row has two values a thread, short chains of loads; many rows fill the chip anyway
+    const int threads = n_out >= 256 ? 256 : width >= 2048 ? 1024 : width >= 1024 ? 512 : 256;
     PALM_DTYPE_SWITCH(d_dtype, TD, {
         PALM_DTYPE_SWITCH(out_dtype, TO,
             add_scaled_normed_kernel<TD, TO><<<n_out, threads, lds, stream>>>(x, (const TD*)d0, c0, (const TD*)d1, c1, ls, w, eps, rows, width,

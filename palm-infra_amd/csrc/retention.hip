@@ -272,7 +272,7 @@ PALM_API int palm_joined_norm_gate(hipStream_t stream, const float* raw, const f
     PALM_CHECK(gate_act == 0 || gate_act == 1, "joined_norm_gate: gate activation %d is neither silu (0) nor sigmoid (1)", gate_act);
     if (n_tokens == 0) return 0;
     PALM_DTYPE_SWITCH(dtype, T,
-        joined_norm_gate_kernel<T><<<n_tokens, width >= 2048 ? 1024 : width >= 1024 ? 512 : 256, 0, stream>>>(raw, weight, eps, (const T*)gate, gate_stride, gate_act, width, (T*)out));
+        joined_norm_gate_kernel<T><<<n_tokens, n_tokens >= 256 ? 256 : width >= 2048 ? 1024 : width >= 1024 ? 512 : 256, 0, stream>>>(raw, weight, eps, (const T*)gate, gate_stride, gate_act, width, (T*)out));
     PALM_LAUNCHED();
     return 0;
 }
