@@ -125,15 +125,16 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
     static constexpr int N = 4;
-    __device__ static void load(const float* p, float (&o)[4]) {
-        const float4 v = *reinterpret_cast<const float4*>(p);
-        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    __device__ static void unpack(const uint4 v, float (&o)[4]) {
+        o[0] = __builtin_bit_cast(float, v.x); o[1] = __builtin_bit_cast(float, v.y);
+        o[2] = __builtin_bit_cast(float, v.z); o[3] = __builtin_bit_cast(float, v.w);
     }
+    __device__ static void load(const float* p, float (&o)[4]) { unpack(*reinterpret_cast<const uint4*>(p), o); }
 };
 template <> struct Vec16<bf16_t> {
     static constexpr int N = 8;
-    __device__ static void load(const bf16_t* p, float (&o)[8]) {
-        const uint4 v = *reinterpret_cast<const uint4*>(p);
+    __device__ static void load(const bf16_t* p, float (&o)[8]) { unpack(*reinterpret_cast<const uint4*>(p), o); }
+    __device__ static void unpack(const uint4 v, float (&o)[8]) {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -204,14 +205,36 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
 #pragma unroll
         for (int qh = 0; qh < MAXQ; ++qh) s[qh] = 0.f;
         const T* kr = kp + (size_t)lane * dim;
+        // 2-byte elements: the lane's rows of the transposed value page (128 bytes each) are all asked for here, before
+        // the scores are made, so that they arrive while the softmax is at work
+        constexpr bool V_AHEAD = sizeof(T) == 2;
+        uint4 vraw[V_AHEAD ? SK_VACC : 1][V_AHEAD ? PAGE_TOKENS / VN : 1];
+        if constexpr (V_AHEAD) {
+#pragma unroll
+            for (int i = 0; i < SK_VACC; ++i) {
+                if (i * WAVE < vdim) {
+                    const T* vr = vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS;
+#pragma unroll
+                    for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) vraw[i][c8] = *reinterpret_cast<const uint4*>(vr + c8 * VN);
+                }
+            }
+        }
         if (k_vec) {
-            for (int d0 = 0; d0 < dim; d0 += VN) {
-                float kv[VN];
-                Vec16<T>::load(kr + d0, kv);
+            // four reads of 16 bytes are under way together (the last ones of a short row repeat its end and are not used)
+            for (int d0 = 0; d0 < dim; d0 += 4 * VN) {
+                uint4 raw[4];
 #pragma unroll
-                for (int e = 0; e < VN; ++e)
+                for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4*>(kr + min(d0 + u * VN, dim - VN));
 #pragma unroll
-                    for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d0 + e], kv[e], s[qh]);
+                for (int u = 0; u < 4; ++u) {
+                    if (d0 + u * VN >= dim) break;
+                    float kv[VN];
+                    Vec16<T>::unpack(raw[u], kv);
+#pragma unroll
+                    for (int e = 0; e < VN; ++e)
+#pragma unroll
+                        for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d0 + u * VN + e], kv[e], s[qh]);
+                }
             }
         } else {
             for (int d = 0; d < dim; ++d) {
@@ -235,6 +258,27 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
         // values: lane c owns columns c, c + 64, ..; its rows of the transposed page are read 16 bytes at a time
         const int j_first = max(lo, pg * PAGE_TOKENS) - pg * PAGE_TOKENS;
         const int j_last = min(pos, pg * PAGE_TOKENS + PAGE_TOKENS - 1) - pg * PAGE_TOKENS;
+        if constexpr (V_AHEAD) {
+#pragma unroll
+            for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) {
+                const int j0 = c8 * VN;
+                if (j0 + VN - 1 < j_first || j0 > j_last) continue;       // (the same in every lane)
+                float vv[SK_VACC][VN];
+#pragma unroll
+                for (int i = 0; i < SK_VACC; ++i)
+                    if (i * WAVE < vdim) Vec16<T>::unpack(vraw[i][c8], vv[i]);
+#pragma unroll
+                for (int e = 0; e < VN; ++e) {
+#pragma unroll
+                    for (int qh = 0; qh < MAXQ; ++qh) {
+                        const float pj = lane_value(p[qh], j0 + e);
+#pragma unroll
+                        for (int i = 0; i < SK_VACC; ++i)
+                            if (i * WAVE < vdim) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
+                    }
+                }
+            }
+        } else
         for (int j0 = j_first / VN * VN; j0 <= j_last; j0 += VN) {
             float vv[SK_VACC][VN];
 #pragma unroll
