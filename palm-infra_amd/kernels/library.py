@@ -29,6 +29,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -173,7 +174,8 @@ def _compile(name: str, sources, defines, force: bool) -> Path:
         shutil.rmtree(work, ignore_errors=True)
     # libraries of older sources are of no use any more
     for old in out.parent.glob(f"libpalm_{name}_*.so"):
-        if old != out:
+        # (of this library only: another library's name may begin with this one's)
+        if old != out and re.fullmatch(rf"libpalm_{re.escape(name)}_[0-9a-f]{{16}}\.so", old.name):
             try:
                 old.unlink()
             except OSError:
