@@ -148,8 +148,9 @@ __device__ inline float lane_value(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
-// Workspace of a (token, head, slice): m, l, then vdim sums.
-template <typename T, int MAXQ>
+// Workspace of a (token, head, slice): m, l, then vdim sums.  NV: value columns a lane (the value size over 64, rounded up),
+// a number of the build so that the innermost loops hold no test.
+template <typename T, int MAXQ, int NV>
 __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int max_pages, const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_new,
@@ -178,14 +179,14 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     }
     __syncthreads();
 
-    float m[MAXQ], l[MAXQ], acc[MAXQ][SK_VACC];
+    float m[MAXQ], l[MAXQ], acc[MAXQ][NV];
 #pragma unroll
     for (int qh = 0; qh < MAXQ; ++qh) {
         const bool sink_here = has_sink && slice == 0 && wave == 0;
         m[qh] = sink_here ? sink_score : -INFINITY;
         l[qh] = sink_here ? 1.f : 0.f;
 #pragma unroll
-        for (int i = 0; i < SK_VACC; ++i) acc[qh][i] = 0.f;
+        for (int i = 0; i < NV; ++i) acc[qh][i] = 0.f;
     }
 
     // this slice's pages
@@ -208,15 +209,13 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
         // 2-byte elements: the lane's rows of the transposed value page (128 bytes each) are all asked for here, before
         // the scores are made, so that they arrive while the softmax is at work
         constexpr bool V_AHEAD = sizeof(T) == 2;
-        uint4 vraw[V_AHEAD ? SK_VACC : 1][V_AHEAD ? PAGE_TOKENS / VN : 1];
+        uint4 vraw[V_AHEAD ? NV : 1][V_AHEAD ? PAGE_TOKENS / VN : 1];
         if constexpr (V_AHEAD) {
 #pragma unroll
-            for (int i = 0; i < SK_VACC; ++i) {
-                if (i * WAVE < vdim) {
-                    const T* vr = vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS;
+            for (int i = 0; i < NV; ++i) {
+                const T* vr = vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS;
 #pragma unroll
-                    for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) vraw[i][c8] = *reinterpret_cast<const uint4*>(vr + c8 * VN);
-                }
+                for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) vraw[i][c8] = *reinterpret_cast<const uint4*>(vr + c8 * VN);
             }
         }
         if (k_vec) {
@@ -253,7 +252,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
             l[qh] = l[qh] * alpha + wave_sum(p[qh]);
             m[qh] = m_new;
 #pragma unroll
-            for (int i = 0; i < SK_VACC; ++i) acc[qh][i] *= alpha;
+            for (int i = 0; i < NV; ++i) acc[qh][i] *= alpha;
         }
         // values: lane c owns columns c, c + 64, ..; its rows of the transposed page are read 16 bytes at a time
         const int j_first = max(lo, pg * PAGE_TOKENS) - pg * PAGE_TOKENS;
@@ -263,37 +262,31 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
             for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) {
                 const int j0 = c8 * VN;
                 if (j0 + VN - 1 < j_first || j0 > j_last) continue;       // (the same in every lane)
-                float vv[SK_VACC][VN];
+                float vv[NV][VN];
 #pragma unroll
-                for (int i = 0; i < SK_VACC; ++i)
-                    if (i * WAVE < vdim) Vec16<T>::unpack(vraw[i][c8], vv[i]);
+                for (int i = 0; i < NV; ++i) Vec16<T>::unpack(vraw[i][c8], vv[i]);
 #pragma unroll
                 for (int e = 0; e < VN; ++e) {
 #pragma unroll
                     for (int qh = 0; qh < MAXQ; ++qh) {
                         const float pj = lane_value(p[qh], j0 + e);
 #pragma unroll
-                        for (int i = 0; i < SK_VACC; ++i)
-                            if (i * WAVE < vdim) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
+                        for (int i = 0; i < NV; ++i) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
                     }
                 }
             }
         } else
         for (int j0 = j_first / VN * VN; j0 <= j_last; j0 += VN) {
-            float vv[SK_VACC][VN];
+            float vv[NV][VN];
 #pragma unroll
-            for (int i = 0; i < SK_VACC; ++i) {
-                const int c = min(lane + i * WAVE, vdim - 1);
-                if (i * WAVE < vdim) Vec16<T>::load(vp + (size_t)c * PAGE_TOKENS + j0, vv[i]);
-            }
+            for (int i = 0; i < NV; ++i) Vec16<T>::load(vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS + j0, vv[i]);
 #pragma unroll
             for (int e = 0; e < VN; ++e) {
 #pragma unroll
                 for (int qh = 0; qh < MAXQ; ++qh) {
                     const float pj = lane_value(p[qh], j0 + e);   // zero for a key that is not seen
 #pragma unroll
-                    for (int i = 0; i < SK_VACC; ++i)
-                        if (i * WAVE < vdim) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
+                    for (int i = 0; i < NV; ++i) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
                 }
             }
         }
@@ -303,7 +296,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     for (int qh = 0; qh < MAXQ; ++qh) {
         if (lane == 0) { m_s[wave][qh] = m[qh]; l_s[wave][qh] = l[qh]; }
 #pragma unroll
-        for (int i = 0; i < SK_VACC; ++i) {
+        for (int i = 0; i < NV; ++i) {
             const int c = lane + i * WAVE;
             if (c < vdim) acc_s[wave][qh][c] = acc[qh][i];
         }
@@ -377,16 +370,19 @@ PALM_API int palm_sink_attention(hipStream_t stream, const void* q, int dtype, c
     PALM_CHECK(kv_heads * chunks <= 65535 && (long long)n_seqs * n_slices <= 65535,
                "sink_attention: %d kv heads / %d sequences x %d slices are more than one launch takes", kv_heads, n_seqs, n_slices);
     dim3 grid(max_new, kv_heads * chunks, n_seqs * n_slices);
-#define SK_CASE(Q) sink_attention_kernel<T, Q><<<grid, SK_WAVES * WAVE, 0, stream>>>((const T*)q, (const T*)k_cache, (const T*)v_cache, \
+    const int nv = (vdim + WAVE - 1) / WAVE;
+#define SK_CASE_V(Q, V) sink_attention_kernel<T, Q, V><<<grid, SK_WAVES * WAVE, 0, stream>>>((const T*)q, (const T*)k_cache, (const T*)v_cache, \
         block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, heads, kv_heads, dim, vdim, scale, window, has_sink, sink_score, \
         (const T*)gate, gate_stride, n_slices, work, (T*)out)
+#define SK_CASE(Q) { if (nv == 1) SK_CASE_V(Q, 1); else if (nv == 2) SK_CASE_V(Q, 2); else if (nv == 3) SK_CASE_V(Q, 3); else SK_CASE_V(Q, 4); }
     PALM_DTYPE_SWITCH(dtype, T, {
-        if (maxq == 1) SK_CASE(1); else if (maxq == 2) SK_CASE(2); else if (maxq == 4) SK_CASE(4); else SK_CASE(8);
+        if (maxq == 1) SK_CASE(1) else if (maxq == 2) SK_CASE(2) else if (maxq == 4) SK_CASE(4) else SK_CASE(8)
         if (n_slices > 1)
             sink_attention_merge_kernel<T><<<dim3(n_tokens, heads), 64, 0, stream>>>(work, n_slices, heads, vdim, (const T*)gate, gate_stride,
                                                                                     (T*)out);
     });
 #undef SK_CASE
+#undef SK_CASE_V
     PALM_LAUNCHED();
     return 0;
 }
