@@ -172,16 +172,20 @@ def _compile(name: str, sources, defines, force: bool) -> Path:
         os.replace(tmp, out)
     finally:
         shutil.rmtree(work, ignore_errors=True)
-    # libraries of older sources are of no use any more
+    remove_older_builds(out, name)
+    _say(f"built {out.name} in {time.time() - t0:.0f} s")
+    return out
+
+
+def remove_older_builds(out: Path, name: str) -> None:
+    """Libraries of older sources are of no use any more: whatever of library ``name`` lies beside ``out`` goes.  Of this
+    library only: another library's name may begin with this one's (``sink_attention`` and ``sink_attention_k2_v4``)."""
     for old in out.parent.glob(f"libpalm_{name}_*.so"):
-        # (of this library only: another library's name may begin with this one's)
         if old != out and re.fullmatch(rf"libpalm_{re.escape(name)}_[0-9a-f]{{16}}\.so", old.name):
             try:
                 old.unlink()
             except OSError:
                 pass
-    _say(f"built {out.name} in {time.time() - t0:.0f} s")
-    return out
 
 
 def _spec(name: str):

@@ -164,3 +164,13 @@ def test_stop_tokens_of_generation_config_join_those_of_config(tmp_path):
     assert config_from_dir(tmp_path).spec().stop_token_ids == (7, 9)
     (tmp_path / "generation_config.json").write_text(json.dumps({"top_k": 20}))
     assert config_from_dir(tmp_path).eos_token_ids == (7,)
+
+
+def test_a_rebuilt_library_removes_its_own_older_builds_only(tmp_path):
+    from palm_infra_amd.kernels.library import remove_older_builds
+    names = ["libpalm_sink_attention_0123456789abcdef.so", "libpalm_sink_attention_fedcba9876543210.so",
+             "libpalm_sink_attention_k2_v4_0123456789abcdef.so", "libpalm_core_0123456789abcdef.so"]
+    for n in names:
+        (tmp_path / n).write_text("")
+    remove_older_builds(tmp_path / names[1], "sink_attention")
+    assert sorted(p.name for p in tmp_path.iterdir()) == sorted(names[1:])

@@ -267,6 +267,11 @@ def test_scaled_add_of_one_and_two_terms_and_the_next_norm(W):
         assert torch.allclose(xd.cpu().double(), x.double() + a_.double(), atol=1e-5)
         empty = ops.add_scaled_normed(xd, [a_.cuda()], [1.0], ls.cuda(), w.cuda(), eps, torch.float32, rows=torch.empty(0, dtype=torch.int32).cuda())
         assert empty.shape == (0, W)
+    # a sum that a part hands back unmade, made by whoever cannot take its terms: three terms, two a pass
+    from palm_infra_amd.parts import WeightedSum, as_tensor
+    c = torch.randn(n, W)
+    total = as_tensor(WeightedSum([a.cuda(), b.cuda(), c.cuda()], [0.5, -1.0, 2.0]))
+    assert total.dtype == torch.float32 and torch.allclose(total.cpu().double(), 0.5 * a.double() - b.double() + 2.0 * c.double(), atol=1e-5)
 
 
 @gpu
