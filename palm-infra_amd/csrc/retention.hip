@@ -96,10 +96,20 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
     {
         const float* at = sp - v + min(v, vdim - 1);
         const bool zero = mode == RET_LOCAL || !mine;
+        if (dim == DMAX) {                                        // the usual case: every row exists, one stride for all reads
+            const size_t stride = (size_t)vdim;
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d) {
-            const float s0 = at[(size_t)min(d, dim - 1) * vdim];
-            S[d] = (zero || d >= dim) ? 0.f : s0;
+            for (int d = 0; d < DMAX; ++d) S[d] = at[d * stride];
+            if (zero) {
+#pragma unroll
+                for (int d = 0; d < DMAX; ++d) S[d] = 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < DMAX; ++d) {
+                const float s0 = at[(size_t)min(d, dim - 1) * vdim];
+                S[d] = (zero || d >= dim) ? 0.f : s0;
+            }
         }
     }
 
@@ -158,9 +168,14 @@ __global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, in
         __syncthreads();
     }
     if (mine && n_new > 0 && mode != RET_FROM_STARTS) {
+        if (dim == DMAX) {
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d)
-            if (d < dim) sp[(size_t)d * vdim] = S[d];
+            for (int d = 0; d < DMAX; ++d) sp[(size_t)d * vdim] = S[d];
+        } else {
+#pragma unroll
+            for (int d = 0; d < DMAX; ++d)
+                if (d < dim) sp[(size_t)d * vdim] = S[d];
+        }
     }
 }
 
