@@ -144,10 +144,6 @@ template <> struct Vec16<bf16_t> {
     }
 };
 
-__device__ inline float lane_value(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-
 // Workspace of a (token, head, slice): m, l, then vdim sums.  NV: value columns a lane (the value size over 64, rounded up),
 // a number of the build so that the innermost loops hold no test.
 template <typename T, int MAXQ, int NV>
@@ -159,6 +155,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     __shared__ float q_s[MAXQ][SK_MAX_DIM];
     __shared__ float m_s[SK_WAVES][MAXQ], l_s[SK_WAVES][MAXQ];
     __shared__ float acc_s[SK_WAVES][MAXQ][SK_MAX_DIM];
+    __shared__ float p_s[SK_WAVES][MAXQ][PAGE_TOKENS];           // a wave's weights of the page at hand, for all its lanes to read
 
     const int per_kv = heads / kv_heads;
     const int chunks = (per_kv + MAXQ - 1) / MAXQ;                 // a group of more than MAXQ heads goes through in several blocks
@@ -184,7 +181,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     for (int qh = 0; qh < MAXQ; ++qh) {
         const bool sink_here = has_sink && slice == 0 && wave == 0;
         m[qh] = sink_here ? sink_score : -INFINITY;
-        l[qh] = sink_here ? 1.f : 0.f;
+        l[qh] = sink_here && lane == 0 ? 1.f : 0.f;              // (a lane's part of the running sum)
 #pragma unroll
         for (int i = 0; i < NV; ++i) acc[qh][i] = 0.f;
     }
@@ -195,6 +192,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     const int s_lo = p_lo + slice * per_slice, s_hi = min(p_hi, s_lo + per_slice - 1);
     constexpr int VN = Vec16<T>::N;
     const bool k_vec = dim % VN == 0;
+    const bool k_full = dim % (4 * VN) == 0, v_full = vdim % WAVE == 0;
 
     for (int pg = s_lo + wave; pg <= s_hi; pg += SK_WAVES) {
         const int page = pages[pg];
@@ -213,13 +211,30 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
         if constexpr (V_AHEAD) {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                const T* vr = vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS;
+                // (a value size of whole waves, the usual case, needs no clamp: plain strides make the cheapest addresses)
+                const T* vr = vp + (size_t)(v_full ? lane + i * WAVE : min(lane + i * WAVE, vdim - 1)) * PAGE_TOKENS;
 #pragma unroll
                 for (int c8 = 0; c8 < PAGE_TOKENS / VN; ++c8) vraw[i][c8] = *reinterpret_cast<const uint4*>(vr + c8 * VN);
             }
         }
-        if (k_vec) {
-            // four reads of 16 bytes are under way together (the last ones of a short row repeat its end and are not used)
+        if (k_full) {
+            // four reads of 16 bytes are under way together
+            for (int d0 = 0; d0 < dim; d0 += 4 * VN) {
+                uint4 raw[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4*>(kr + d0 + u * VN);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    float kv[VN];
+                    Vec16<T>::unpack(raw[u], kv);
+#pragma unroll
+                    for (int e = 0; e < VN; ++e)
+#pragma unroll
+                        for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d0 + u * VN + e], kv[e], s[qh]);
+                }
+            }
+        } else if (k_vec) {
+            // (the last reads of a row that is no multiple of four reads repeat its end and are not used)
             for (int d0 = 0; d0 < dim; d0 += 4 * VN) {
                 uint4 raw[4];
 #pragma unroll
@@ -242,18 +257,36 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
                 for (int qh = 0; qh < MAXQ; ++qh) s[qh] = fmaf(q_s[qh][d], kd, s[qh]);
             }
         }
-        float p[MAXQ];
+        // the page's maxima of all heads together: every step's exchanges between lanes are under way at once
+        float p[MAXQ], top[MAXQ];
+#pragma unroll
+        for (int qh = 0; qh < MAXQ; ++qh) top[qh] = s[qh] = seen ? s[qh] : -INFINITY;
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) {
+            float other[MAXQ];
+#pragma unroll
+            for (int qh = 0; qh < MAXQ; ++qh) other[qh] = __shfl_xor(top[qh], off, WAVE);
+#pragma unroll
+            for (int qh = 0; qh < MAXQ; ++qh) top[qh] = fmaxf(top[qh], other[qh]);
+        }
 #pragma unroll
         for (int qh = 0; qh < MAXQ; ++qh) {
-            const float sc = seen ? s[qh] : -INFINITY;
-            const float m_new = fmaxf(m[qh], wave_max(sc));       // every page of the range holds a key that is seen
+            const float m_new = fmaxf(m[qh], top[qh]);            // every page of the range holds a key that is seen
             const float alpha = expf(m[qh] - m_new);              // m = -inf at the first page: exp(-inf) = 0
-            p[qh] = expf(sc - m_new);                             // a key that is not seen: exp(-inf) = 0
-            l[qh] = l[qh] * alpha + wave_sum(p[qh]);
+            p[qh] = expf(s[qh] - m_new);                          // a key that is not seen: exp(-inf) = 0
+            l[qh] = l[qh] * alpha + p[qh];                        // this lane's part of the sum; the lanes are added at the end
             m[qh] = m_new;
 #pragma unroll
             for (int i = 0; i < NV; ++i) acc[qh][i] *= alpha;
         }
+        // A lane holds the weight of its key; every lane needs every key's.  They go through LDS (all lanes read one
+        // address: one pass), four keys a read, which costs far less than handing them out lane by lane as scalars.
+        // The wave's own reads follow its own writes in order; the fences keep the compiler from moving them.
+#pragma unroll
+        for (int qh = 0; qh < MAXQ; ++qh) p_s[wave][qh][lane] = p[qh];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // values: lane c owns columns c, c + 64, ..; its rows of the transposed page are read 16 bytes at a time
         const int j_first = max(lo, pg * PAGE_TOKENS) - pg * PAGE_TOKENS;
         const int j_last = min(pos, pg * PAGE_TOKENS + PAGE_TOKENS - 1) - pg * PAGE_TOKENS;
@@ -266,10 +299,10 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
 #pragma unroll
                 for (int i = 0; i < NV; ++i) Vec16<T>::unpack(vraw[i][c8], vv[i]);
 #pragma unroll
-                for (int e = 0; e < VN; ++e) {
+                for (int qh = 0; qh < MAXQ; ++qh) {
 #pragma unroll
-                    for (int qh = 0; qh < MAXQ; ++qh) {
-                        const float pj = lane_value(p[qh], j0 + e);
+                    for (int e = 0; e < VN; ++e) {
+                        const float pj = p_s[wave][qh][j0 + e];
 #pragma unroll
                         for (int i = 0; i < NV; ++i) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
                     }
@@ -281,20 +314,23 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
 #pragma unroll
             for (int i = 0; i < NV; ++i) Vec16<T>::load(vp + (size_t)min(lane + i * WAVE, vdim - 1) * PAGE_TOKENS + j0, vv[i]);
 #pragma unroll
-            for (int e = 0; e < VN; ++e) {
+            for (int qh = 0; qh < MAXQ; ++qh) {
 #pragma unroll
-                for (int qh = 0; qh < MAXQ; ++qh) {
-                    const float pj = lane_value(p[qh], j0 + e);   // zero for a key that is not seen
+                for (int e = 0; e < VN; ++e) {
+                    const float pj = p_s[wave][qh][j0 + e];       // zero for a key that is not seen
 #pragma unroll
                     for (int i = 0; i < NV; ++i) acc[qh][i] = fmaf(pj, vv[i][e], acc[qh][i]);
                 }
             }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // (the next page's weights are written after these reads)
+        __builtin_amdgcn_wave_barrier();
     }
 
 #pragma unroll
     for (int qh = 0; qh < MAXQ; ++qh) {
-        if (lane == 0) { m_s[wave][qh] = m[qh]; l_s[wave][qh] = l[qh]; }
+        const float l_wave = wave_sum(l[qh]);
+        if (lane == 0) { m_s[wave][qh] = m[qh]; l_s[wave][qh] = l_wave; }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = lane + i * WAVE;
