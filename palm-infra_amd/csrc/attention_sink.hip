@@ -13,8 +13,9 @@
 // exact kernel (32-bit arithmetic), which serves the float32 mode, single tokens, and whatever the matrix-core kernel
 // does not take.  One block of four waves per (query, group of up to eight query heads that share a key/value head,
 // slice of the key range): a key or value is read once for all those heads.  A wave takes every fourth page of the
-// slice; in a page each lane scores one key for all heads, the wave keeps a running (max, sum, output) for each head,
-// and the four waves' partial results are merged at the end.  With one slice the block then gates and writes the
+// slice; in a page each lane scores one key for all heads and owns a few value columns (the weights reach all lanes
+// through LDS), the wave keeps a running (max, sum, output) for each head, and the four waves' partial results are
+// merged at the end.  With one slice the block then gates and writes the
 // output; with more (a decode step: few queries over long ranges) it leaves its partial result in a workspace for
 // the merging kernel.
 #include "common.h"
