@@ -361,26 +361,39 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     }
 }
 
-// The slices of a (token, head) merged, gated and written.
+// The slices of a (token, head) merged, gated and written: one wave.  The slices' maxima and sums are read a slice a lane
+// (all reads under way at once), their weights wait in LDS, and the columns' sums run over the slices four reads at a time.
+constexpr int SK_MAX_SLICES = 1024;
+
 template <typename T>
-__global__ void sink_attention_merge_kernel(const float* __restrict__ work, int n_slices, int heads, int vdim, const T* __restrict__ gate,
-                                            int gate_stride, T* __restrict__ out) {
+__global__ __launch_bounds__(WAVE) void sink_attention_merge_kernel(const float* __restrict__ work, int n_slices, int heads, int vdim,
+                                                                    const T* __restrict__ gate, int gate_stride, T* __restrict__ out) {
+    __shared__ float w_s[SK_MAX_SLICES];
     const size_t t = blockIdx.x;
-    const int h = blockIdx.y;
-    const float* wk = work + ((t * heads + h) * n_slices) * (size_t)(vdim + 2);
-    float m_all = -INFINITY;
-    for (int s = 0; s < n_slices; ++s) m_all = fmaxf(m_all, wk[(size_t)s * (vdim + 2)]);
-    float l_all = 0.f;
-    for (int s = 0; s < n_slices; ++s) {
-        const float ms = wk[(size_t)s * (vdim + 2)];
-        l_all += ms == -INFINITY ? 0.f : wk[(size_t)s * (vdim + 2) + 1] * expf(ms - m_all);
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const size_t stride = (size_t)(vdim + 2);
+    const float* wk = work + ((t * heads + h) * n_slices) * stride;
+    float m_loc = -INFINITY;
+    for (int s = lane; s < n_slices; s += WAVE) m_loc = fmaxf(m_loc, wk[s * stride]);
+    const float m_all = wave_max(m_loc);
+    float l_loc = 0.f;
+    for (int s = lane; s < n_slices; s += WAVE) {
+        const float ms = wk[s * stride];
+        const float w = ms == -INFINITY ? 0.f : expf(ms - m_all);
+        w_s[s] = w;
+        l_loc = fmaf(wk[s * stride + 1], w, l_loc);
     }
-    for (int c = threadIdx.x; c < vdim; c += blockDim.x) {
+    const float l_all = wave_sum(l_loc);
+    __syncthreads();
+    for (int c = lane; c < vdim; c += WAVE) {
+        const float* col = wk + 2 + c;
         float o = 0.f;
-        for (int s = 0; s < n_slices; ++s) {
-            const float ms = wk[(size_t)s * (vdim + 2)];
-            if (ms != -INFINITY) o += wk[(size_t)s * (vdim + 2) + 2 + c] * expf(ms - m_all);
+        int s = 0;
+        for (; s + 4 <= n_slices; s += 4) {
+            const float a0 = col[(s + 0) * stride], a1 = col[(s + 1) * stride], a2 = col[(s + 2) * stride], a3 = col[(s + 3) * stride];
+            o = fmaf(a0, w_s[s], o); o = fmaf(a1, w_s[s + 1], o); o = fmaf(a2, w_s[s + 2], o); o = fmaf(a3, w_s[s + 3], o);
         }
+        for (; s < n_slices; ++s) o = fmaf(col[s * stride], w_s[s], o);
         float r = o / l_all;
         if (gate) { const float gt = to_float(gate[t * gate_stride + (size_t)h * vdim + c]); r *= 1.0f / (1.0f + expf(-gt)); }
         out[(t * heads + h) * vdim + c] = from_float<T>(r);
@@ -399,7 +412,8 @@ PALM_API int palm_sink_attention(hipStream_t stream, const void* q, int dtype, c
     PALM_CHECK(heads % kv_heads == 0, "sink_attention: %d heads are not a multiple of %d kv heads", heads, kv_heads);
     PALM_CHECK(dim <= SK_MAX_DIM && vdim <= SK_MAX_DIM, "sink_attention: key size %d / value size %d exceed %d", dim, vdim, SK_MAX_DIM);
     PALM_CHECK(window >= 0 && max_pages > 0, "sink_attention: window %d, max_pages %d", window, max_pages);
-    PALM_CHECK(n_slices >= 1 && (n_slices == 1 || work), "sink_attention: %d slices need a workspace", n_slices);
+    PALM_CHECK(n_slices >= 1 && n_slices <= SK_MAX_SLICES && (n_slices == 1 || work), "sink_attention: %d slices (at most %d) need a workspace",
+               n_slices, SK_MAX_SLICES);
     if (n_seqs == 0 || max_new == 0 || n_tokens == 0) return 0;
     const int per_kv = heads / kv_heads;
     const int maxq = per_kv >= 8 ? 8 : per_kv > 2 ? 4 : per_kv;
