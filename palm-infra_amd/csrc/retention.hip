@@ -260,6 +260,23 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
     return 0;
 }
 
+__device__ inline void ret_load4(const float* p, float (&o)[4]) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ inline void ret_load4(const bf16_t* p, float (&o)[4]) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    o[0] = __builtin_bit_cast(float, v.x << 16); o[1] = __builtin_bit_cast(float, v.x & 0xffff0000u);
+    o[2] = __builtin_bit_cast(float, v.y << 16); o[3] = __builtin_bit_cast(float, v.y & 0xffff0000u);
+}
+__device__ inline void ret_store4(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ inline void ret_store4(bf16_t* p, const float (&v)[4]) {
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+    w.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
 // ---- the joined heads normed together and gated -------------------------------------------------------------
 // out[t] = raw[t] / sqrt(mean(raw[t]^2) + eps) * weight * f(gate[t]) over a token's whole row of `width` values (all
 // heads), f = sigmoid (gate_act 1) or silu (gate_act 0).  raw is 32-bit; the gate lies in rows `gate_stride` elements
@@ -272,12 +289,32 @@ __global__ __launch_bounds__(1024) void joined_norm_gate_kernel(const float* __r
     const size_t t = blockIdx.x;
     const float* r = raw + t * width;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) { const float v = r[c]; ss += v * v; }
+    // four values a read where the row and the gate's rows allow
+    const bool by_four = width % 4 == 0 && gate_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(gate) % 16) == 0;
+    if (by_four) {
+        for (int c = threadIdx.x * 4; c < width; c += blockDim.x * 4) {
+            const float4 v = *reinterpret_cast<const float4*>(r + c);
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    } else {
+        for (int c = threadIdx.x; c < width; c += blockDim.x) { const float v = r[c]; ss += v * v; }
+    }
     const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
-        const float g = to_float(gate[t * gate_stride + c]);
+    auto gated = [&](float o, float w, float g) {
         const float f = gate_act == 1 ? 1.0f / (1.0f + expf(-g)) : g / (1.0f + expf(-g));
-        out[t * width + c] = from_float<T>(r[c] * inv * weight[c] * f);
+        return o * inv * w * f;
+    };
+    if (by_four) {
+        for (int c = threadIdx.x * 4; c < width; c += blockDim.x * 4) {
+            const float4 v = *reinterpret_cast<const float4*>(r + c), w = *reinterpret_cast<const float4*>(weight + c);
+            float g[4];
+            ret_load4(gate + t * gate_stride + c, g);
+            const float y[4] = {gated(v.x, w.x, g[0]), gated(v.y, w.y, g[1]), gated(v.z, w.z, g[2]), gated(v.w, w.w, g[3])};
+            ret_store4(out + t * width + c, y);
+        }
+    } else {
+        for (int c = threadIdx.x; c < width; c += blockDim.x)
+            out[t * width + c] = from_float<T>(gated(r[c], weight[c], to_float(gate[t * gate_stride + c])));
     }
 }
 
