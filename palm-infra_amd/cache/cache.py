@@ -261,8 +261,14 @@ class ModelCache:
                     raise ValueError(f"run-order entry {i}: {e}") from None
         for i, src in enumerate(shares):
             if src is not None:
-                self.layer_caches[i] = copy.copy(self.layer_caches[src])      # whatever its groups hung on it
-                self.layer_caches[i].writes = False
+                own = self.layer_caches[i]                                    # what the entry keeps beside what it reads
+                if own.kv is not None:
+                    raise ValueError(f"run-order entry {i} reads the keys and values of entry {src} and asks for some of its own")
+                merged = copy.copy(self.layer_caches[src])                    # whatever the source's groups hung on it
+                merged.writes = False
+                merged.states = {**(merged.states or {}), **(own.states or {})} or None
+                merged.rows = {**(merged.rows or {}), **(own.rows or {})} or None
+                self.layer_caches[i] = merged
 
     def groups_of(self, need_type) -> list:
         """The groups whose need is of the given class, in the order in which the run order first asked for them."""

@@ -6,8 +6,9 @@ from .qwen3 import Qwen3Config
 from .sebesun import SebesunConfig
 from .pazilorn import PazilornConfig
 from .matalix import MatalixConfig
+from .biguzen import BiguzenConfig
 
 __all__ = ["ConfigError", "config_class_for", "config_from_dict", "config_from_dir", "config_source", "preset_dict",
            "preset_names", "register_architecture",
            "registered_architectures", "LayerCall", "ModelSpec", "PartSpec", "Stored", "TensorRef", "joined", "tensor",
-           "Qwen3Config", "SebesunConfig", "PazilornConfig", "MatalixConfig"]
+           "Qwen3Config", "SebesunConfig", "PazilornConfig", "MatalixConfig", "BiguzenConfig"]

@@ -58,6 +58,8 @@ class TensorRef:
             raise ValueError(f"TensorRef role {self.role!r} is not one of {ROLES}")
         if len(self.names) != len(self.shapes) or not self.names:
             raise ValueError("TensorRef needs one shape for each name")
+        if len(self.names) > 1 and any(not s for s in self.shapes):
+            raise ValueError(f"tensors {self.names}: single numbers have no rows to be joined along")
         tail = self.shapes[0][1:]
         if any(s[1:] != tail for s in self.shapes):
             raise ValueError(f"tensors {self.names} cannot be joined along rows: shapes {self.shapes}")
@@ -71,6 +73,8 @@ class TensorRef:
 
     @property
     def shape(self) -> tuple[int, ...]:
+        if len(self.shapes) == 1 and not self.shapes[0]:
+            return ()                                   # a single number (a norm's slope): nothing to join
         rows = sum(s[0] for s in self.shapes)
         return (rows,) + tuple(self.shapes[0][1:])
 
@@ -141,11 +145,16 @@ class ModelSpec:
     stop_token_ids: tuple[int, ...] = ()
     # layers read the results of all layers before them (and the embedding's rows): the model keeps them for the step
     keeps_results: bool = False
+    # the residual stream runs in this many copies [n, streams, width], all equal to the embedding's rows at the start; the
+    # blocks and the final norm then read and write streams (None: one stream [n, width])
+    streams: int | None = None
 
     def __post_init__(self):
         for i, call in enumerate(self.order):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"run order entry {i} names layer {call.layer}; there are {len(self.layers)}")
+            if self.streams is not None and (call.adds_embedding or self.keeps_results):
+                raise ValueError("a stream in several copies neither takes the embedding's rows again nor keeps the layers' results")
             if call.cache_of is not None:
                 if not 0 <= call.cache_of < i:
                     raise ValueError(f"run order entry {i} reads the cache of entry {call.cache_of}, "

@@ -2,7 +2,10 @@
 // have: a key size and a value size of their own, an RMS norm over the whole q projection and the whole k projection
 // (or per head, or none), biases on q, k and v, a rotation of the first `rot` dimensions of each head, a sliding
 // window, a sink (a key of a fixed score without a value: it only adds exp(score) to the softmax's denominator), and an
-// elementwise sigmoid gate on the heads' outputs.
+// elementwise sigmoid gate on the heads' outputs (or one gate value for each head).  The sink's score is one number for
+// all heads or a learned one for each.  Between the bias and the norm q, k and v may go through a short causal convolution
+// over time, a channel at a time: y_t = sum_j w[c][j] u_(t - taps + 1 + j) with zeros before the sequence's start; the last
+// taps - 1 inputs u of each sequence are kept as state.  The rotation pairs dimension i with i + rot/2, or 2i with 2i + 1.
 //
 //   p_j = exp(s_j) / (exp(sink) + sum_i exp(s_i)),   s_j = scale * q . k_j,   max(0, pos - window + 1) <= j <= pos
 //   out = (sum_j p_j v_j) * sigmoid(gate)
@@ -36,7 +39,8 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ tok_slot, const int* __restrict__ positions, int norm_mode, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
-    int heads, int kv_heads, int dim, int vdim, int write_cache) {
+    int heads, int kv_heads, int dim, int vdim, int write_cache, int pairing,
+    const float* __restrict__ conv_w, int taps, const float* __restrict__ conv_state, int conv_channels) {
     __shared__ float scratch[16];
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
@@ -46,11 +50,33 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
     const int pos = positions[t];
     const int page = write_cache ? block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS] : 0;
     const int at = pos % PAGE_TOKENS;
+    // The convolution's inputs: of the rows right before this one, `before` belong to the same sequence (a sequence's rows lie
+    // together); what lies further back comes from the sequence's state, oldest first, zero for a sequence that has just begun.
+    int before = 0;
+    const float* st = nullptr;
+    if (taps > 1) {
+        const int slot = tok_slot[t];
+        while (before < taps - 1 && t > (size_t)before && tok_slot[t - before - 1] == slot) ++before;
+        st = conv_state + (size_t)slot * (taps - 1) * conv_channels;
+    }
+    // column `col` of the rows, which is channel `ch` of q | k | v, with its bias, through the convolution
+    auto value = [&](int col, int ch, const float* b) {
+        const float bias_c = b ? *b : 0.f;
+        if (taps <= 1) return to_float(row[col]) + bias_c;
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int back = taps - 1 - j;
+            const float u = back <= before ? to_float(rows[(t - back) * stride + col]) + bias_c
+                                           : st[(size_t)(taps - 1 - (back - before)) * conv_channels + ch];
+            acc = fmaf(conv_w[(size_t)ch * taps + j], u, acc);
+        }
+        return acc;
+    };
     float inv_q = 1.f, inv_k = 1.f;
     if (norm_mode == SK_NORM_PROJECTION) {
         float sq = 0.f, sk = 0.f;
-        for (int i = threadIdx.x; i < q_size; i += blockDim.x) { const float v = to_float(row[q_off + i]) + (q_b ? q_b[i] : 0.f); sq += v * v; }
-        for (int i = threadIdx.x; i < k_size; i += blockDim.x) { const float v = to_float(row[k_off + i]) + (k_b ? k_b[i] : 0.f); sk += v * v; }
+        for (int i = threadIdx.x; i < q_size; i += blockDim.x) { const float v = value(q_off + i, i, q_b ? q_b + i : nullptr); sq += v * v; }
+        for (int i = threadIdx.x; i < k_size; i += blockDim.x) { const float v = value(k_off + i, q_size + i, k_b ? k_b + i : nullptr); sk += v * v; }
         sq = block_sum(sq, scratch);
         sk = block_sum(sk, scratch);
         inv_q = 1.0f / sqrtf(sq / (float)q_size + eps);
@@ -61,7 +87,7 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
         const bool is_q = r < heads;
         if (!is_q && !write_cache) continue;
         const int hh = is_q ? r : r - heads;
-        const T* src = row + (is_q ? q_off : k_off) + (size_t)hh * dim;
+        const int col0 = (is_q ? q_off : k_off) + hh * dim, ch0 = (is_q ? 0 : q_size) + hh * dim;
         const float* b = is_q ? (q_b ? q_b + (size_t)hh * dim : nullptr) : (k_b ? k_b + (size_t)hh * dim : nullptr);
         float inv = is_q ? inv_q : inv_k;
         const float* w = nullptr;
@@ -69,39 +95,71 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
         if (norm_mode == SK_NORM_HEAD) {
             w = is_q ? q_w : k_w;
             float ss = 0.f;
-            for (int d = lane; d < dim; d += WAVE) { const float v = to_float(src[d]) + (b ? b[d] : 0.f); ss += v * v; }
+            for (int d = lane; d < dim; d += WAVE) { const float v = value(col0 + d, ch0 + d, b ? b + d : nullptr); ss += v * v; }
             inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
         }
         T* dst = is_q ? q_out + (t * heads + hh) * dim
                       : k_cache + (((size_t)page * kv_heads + hh) * PAGE_TOKENS + at) * dim;
         auto normed = [&](int d) {
-            const float v = (to_float(src[d]) + (b ? b[d] : 0.f)) * inv;
+            const float v = value(col0 + d, ch0 + d, b ? b + d : nullptr) * inv;
             return w ? v * w[d] : v;
         };
         for (int d = lane; d < dim; d += WAVE) {
             float v = normed(d);
             if (d < rot) {
-                const int i = d < half ? d : d - half;
+                // pairs (i, i + rot/2), or neighbours (2i, 2i + 1)
+                const bool first = pairing == 1 ? (d & 1) == 0 : d < half;
+                const int i = pairing == 1 ? d >> 1 : (d < half ? d : d - half);
+                const int partner = pairing == 1 ? d ^ 1 : (d < half ? d + half : d - half);
                 const float c = cos_t[t * half + i], sn = sin_t[t * half + i];
-                const float pv = normed(d < half ? d + half : d - half);
+                const float pv = normed(partner);
                 // the pair (u, w) becomes (u c - w s, w c + u s)
-                v = d < half ? v * c - pv * sn : v * c + pv * sn;
+                v = first ? v * c - pv * sn : v * c + pv * sn;
             }
             dst[d] = from_float<T>(v);
         }
     }
     if (write_cache) {
-        const T* vs = row + v_off;
         for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x)
-            v_cache[((size_t)page * kv_heads * vdim + i) * PAGE_TOKENS + at] = from_float<T>(to_float(vs[i]) + (v_b ? v_b[i] : 0.f));
+            v_cache[((size_t)page * kv_heads * vdim + i) * PAGE_TOKENS + at] = from_float<T>(value(v_off + i, q_size + k_size + i, v_b ? v_b + i : nullptr));
     }
+}
+
+// After the pass above has read the old state: the last taps - 1 inputs (projection plus bias) of each sequence, old ones
+// moved up.  One thread per (channel, sequence); a thread reads all it keeps before it writes.
+constexpr int SK_MAX_TAPS = 16;
+
+template <typename T>
+__global__ void sink_conv_state_kernel(const T* __restrict__ rows, int stride, int q_off, int k_off, int v_off, int q_size, int k_size,
+                                       const float* __restrict__ bias, float* __restrict__ conv_state, const int* __restrict__ seq_slot,
+                                       const int* __restrict__ seq_new, const int* __restrict__ cu_new, int channels, int taps) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (c >= channels) return;
+    const int n_new = seq_new[b];
+    if (n_new <= 0) return;
+    const int col = c < q_size ? q_off + c : c < q_size + k_size ? k_off + (c - q_size) : v_off + (c - q_size - k_size);
+    const float bias_c = bias ? bias[c] : 0.f;
+    const size_t row0 = (size_t)cu_new[b];
+    float* st = conv_state + (size_t)seq_slot[b] * (taps - 1) * channels;
+    float keep[SK_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < SK_MAX_TAPS; ++j) {
+        if (j < taps - 1) {
+            const int at = n_new - (taps - 1) + j;
+            keep[j] = at >= 0 ? to_float(rows[(row0 + at) * stride + col]) + bias_c : st[(size_t)(taps - 1 + at) * channels + c];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < SK_MAX_TAPS; ++j)
+        if (j < taps - 1) st[(size_t)j * channels + c] = keep[j];
 }
 
 PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype, int stride, int q_off, int k_off, int v_off,
                                  const float* bias, void* q_out, void* k_cache, void* v_cache, const int* block_table, int max_pages,
                                  const int* tok_slot, const int* positions, int norm_mode, const float* q_w, const float* k_w, float eps,
                                  const float* cos_t, const float* sin_t, int rot, int n_tokens, int heads, int kv_heads, int dim, int vdim,
-                                 int write_cache) {
+                                 int write_cache, int pairing, const float* conv_w, int taps, float* conv_state, const int* seq_slot,
+                                 const int* seq_new, const int* cu_new, int n_seqs) {
     PALM_CHECK(n_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "sink_qkv_store: tokens=%d heads=%d kv=%d dim=%d vdim=%d",
                n_tokens, heads, kv_heads, dim, vdim);
     PALM_CHECK(norm_mode >= SK_NORM_NONE && norm_mode <= SK_NORM_HEAD, "sink_qkv_store: norm mode %d", norm_mode);
@@ -109,14 +167,25 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
     PALM_CHECK(rot >= 0 && rot <= dim && rot % 2 == 0, "sink_qkv_store: %d rotated dimensions of %d", rot, dim);
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "sink_qkv_store: a rotation needs its cos and sin rows");
     PALM_CHECK(!write_cache || (k_cache && v_cache && block_table && tok_slot && max_pages > 0), "sink_qkv_store: writing needs cache, pages and slots");
+    PALM_CHECK(pairing == 0 || pairing == 1, "sink_qkv_store: pairing %d is neither halves (0) nor neighbours (1)", pairing);
+    PALM_CHECK(taps >= 0 && taps <= SK_MAX_TAPS, "sink_qkv_store: %d taps (at most %d)", taps, SK_MAX_TAPS);
+    PALM_CHECK(taps <= 1 || (conv_w && conv_state && tok_slot && seq_slot && seq_new && cu_new && n_seqs > 0 && n_seqs <= 65535),
+               "sink_qkv_store: a convolution needs its weights, its state and the step's sequences");
     if (n_tokens == 0) return 0;
+    // the convolution's channels: q, and k and v if this layer makes them
+    const int conv_channels = heads * dim + (write_cache ? kv_heads * (dim + vdim) : 0);
     // a wave takes a head at a time: for few tokens (a decode step) as many waves as there are heads of q and k, within a
     // block's sixteen; many tokens fill the chip anyway
     const int threads = n_tokens >= 256 ? 256 : min(1024, max(256, WAVE * (heads + kv_heads)));
     PALM_DTYPE_SWITCH(dtype, T,
         sink_qkv_store_kernel<T><<<n_tokens, threads, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
                                                               (T*)v_cache, block_table, max_pages, tok_slot, positions, norm_mode, q_w, k_w,
-                                                              eps, cos_t, sin_t, rot, heads, kv_heads, dim, vdim, write_cache));
+                                                              eps, cos_t, sin_t, rot, heads, kv_heads, dim, vdim, write_cache, pairing,
+                                                              conv_w, taps, conv_state, conv_channels);
+        if (taps > 1)
+            sink_conv_state_kernel<T><<<dim3((conv_channels + 255) / 256, n_seqs), 256, 0, stream>>>(
+                (const T*)rows, stride, q_off, k_off, v_off, heads * dim, kv_heads * dim, bias, conv_state, seq_slot, seq_new, cu_new,
+                conv_channels, taps));
     PALM_LAUNCHED();
     return 0;
 }
@@ -152,7 +221,8 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int max_pages, const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_new,
     const int* __restrict__ cu_new, int heads, int kv_heads, int dim, int vdim, float scale, int window, int has_sink,
-    float sink_score, const T* __restrict__ gate, int gate_stride, int n_slices, float* __restrict__ work, T* __restrict__ out) {
+    float sink_score, const float* __restrict__ sink_scores, const T* __restrict__ gate, int gate_stride, int gate_per_head, int n_slices,
+    float* __restrict__ work, T* __restrict__ out) {
     __shared__ float q_s[MAXQ][SK_MAX_DIM];
     __shared__ float m_s[SK_WAVES][MAXQ], l_s[SK_WAVES][MAXQ];
     __shared__ float acc_s[SK_WAVES][MAXQ][SK_MAX_DIM];
@@ -181,7 +251,8 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
 #pragma unroll
     for (int qh = 0; qh < MAXQ; ++qh) {
         const bool sink_here = has_sink && slice == 0 && wave == 0;
-        m[qh] = sink_here ? sink_score : -INFINITY;
+        // one score for all heads, or a learned one for each
+        m[qh] = sink_here ? (sink_scores ? sink_scores[min(h0 + qh, heads - 1)] : sink_score) : -INFINITY;
         l[qh] = sink_here && lane == 0 ? 1.f : 0.f;              // (a lane's part of the running sum)
 #pragma unroll
         for (int i = 0; i < NV; ++i) acc[qh][i] = 0.f;
@@ -351,7 +422,7 @@ __global__ __launch_bounds__(SK_WAVES * WAVE) void sink_attention_kernel(
         }
         if (n_slices == 1) {
             float r = o / l_all;
-            if (gate) { const float gt = to_float(gate[(size_t)t * gate_stride + (size_t)h * vdim + c]); r *= 1.0f / (1.0f + expf(-gt)); }
+            if (gate) { const float gt = to_float(gate[(size_t)t * gate_stride + (gate_per_head ? h : (size_t)h * vdim + c)]); r *= 1.0f / (1.0f + expf(-gt)); }
             out[((size_t)t * heads + h) * vdim + c] = from_float<T>(r);
         } else {
             float* wk = work + (((size_t)t * heads + h) * n_slices + slice) * (vdim + 2);
@@ -367,7 +438,8 @@ constexpr int SK_MAX_SLICES = 1024;
 
 template <typename T>
 __global__ __launch_bounds__(WAVE) void sink_attention_merge_kernel(const float* __restrict__ work, int n_slices, int heads, int vdim,
-                                                                    const T* __restrict__ gate, int gate_stride, T* __restrict__ out) {
+                                                                    const T* __restrict__ gate, int gate_stride, int gate_per_head,
+                                                                    T* __restrict__ out) {
     __shared__ float w_s[SK_MAX_SLICES];
     const size_t t = blockIdx.x;
     const int h = blockIdx.y, lane = threadIdx.x;
@@ -395,18 +467,18 @@ __global__ __launch_bounds__(WAVE) void sink_attention_merge_kernel(const float*
         }
         for (; s < n_slices; ++s) o = fmaf(col[s * stride], w_s[s], o);
         float r = o / l_all;
-        if (gate) { const float gt = to_float(gate[t * gate_stride + (size_t)h * vdim + c]); r *= 1.0f / (1.0f + expf(-gt)); }
+        if (gate) { const float gt = to_float(gate[t * gate_stride + (gate_per_head ? h : (size_t)h * vdim + c)]); r *= 1.0f / (1.0f + expf(-gt)); }
         out[(t * heads + h) * vdim + c] = from_float<T>(r);
     }
 }
 
 // q [n, heads, dim]; gate: null, or the first gate value of token 0 (rows `gate_stride` elements apart, heads * vdim
-// values a row); work: room for n_tokens * heads * n_slices * (vdim + 2) floats if n_slices > 1; out [n, heads * vdim].
+// values a row, or with gate_per_head one value for each head); sink_scores: null, or a score for each head; work: room for n_tokens * heads * n_slices * (vdim + 2) floats if n_slices > 1; out [n, heads * vdim].
 PALM_API int palm_sink_attention(hipStream_t stream, const void* q, int dtype, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* seq_slot, const int* seq_start, const int* seq_new,
                                  const int* cu_new, int n_seqs, int max_new, int n_tokens, int heads, int kv_heads, int dim, int vdim,
-                                 float scale, int window, int has_sink, float sink_score, const void* gate, int gate_stride, int n_slices,
-                                 float* work, void* out) {
+                                 float scale, int window, int has_sink, float sink_score, const float* sink_scores, const void* gate,
+                                 int gate_stride, int gate_per_head, int n_slices, float* work, void* out) {
     PALM_CHECK(n_seqs >= 0 && max_new >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0,
                "sink_attention: seqs=%d max_new=%d heads=%d kv=%d dim=%d vdim=%d", n_seqs, max_new, heads, kv_heads, dim, vdim);
     PALM_CHECK(heads % kv_heads == 0, "sink_attention: %d heads are not a multiple of %d kv heads", heads, kv_heads);
@@ -424,13 +496,13 @@ PALM_API int palm_sink_attention(hipStream_t stream, const void* q, int dtype, c
     const int nv = (vdim + WAVE - 1) / WAVE;
 #define SK_CASE_V(Q, V) sink_attention_kernel<T, Q, V><<<grid, SK_WAVES * WAVE, 0, stream>>>((const T*)q, (const T*)k_cache, (const T*)v_cache, \
         block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, heads, kv_heads, dim, vdim, scale, window, has_sink, sink_score, \
-        (const T*)gate, gate_stride, n_slices, work, (T*)out)
+        sink_scores, (const T*)gate, gate_stride, gate_per_head, n_slices, work, (T*)out)
 #define SK_CASE(Q) { if (nv == 1) SK_CASE_V(Q, 1); else if (nv == 2) SK_CASE_V(Q, 2); else if (nv == 3) SK_CASE_V(Q, 3); else SK_CASE_V(Q, 4); }
     PALM_DTYPE_SWITCH(dtype, T, {
         if (maxq == 1) SK_CASE(1) else if (maxq == 2) SK_CASE(2) else if (maxq == 4) SK_CASE(4) else SK_CASE(8)
         if (n_slices > 1)
             sink_attention_merge_kernel<T><<<dim3(n_tokens, heads), 64, 0, stream>>>(work, n_slices, heads, vdim, (const T*)gate, gate_stride,
-                                                                                    (T*)out);
+                                                                                    gate_per_head, (T*)out);
     });
 #undef SK_CASE
 #undef SK_CASE_V

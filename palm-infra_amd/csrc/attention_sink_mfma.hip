@@ -41,8 +41,10 @@ __global__ __launch_bounds__(WAVE) void sink_attention_mfma_kernel(
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new,
     int heads, int kv_heads, int dim, int vdim, float scale, int window, int has_sink, float sink_score,
-    const bf16_t* __restrict__ gate, int gate_stride, bf16_t* __restrict__ out) {
+    const float* __restrict__ sink_scores, const bf16_t* __restrict__ gate, int gate_stride, int gate_per_head,
+    bf16_t* __restrict__ out) {
     const int h = blockIdx.y, b = blockIdx.z;
+    if (sink_scores) sink_score = sink_scores[h];                 // a learned score for each head instead of one for all
     const int n_new = seq_new[b];
     const int lane = threadIdx.x;
     // the wave's first query among the sequence's new tokens; the blocks of late queries, which have the most keys before
@@ -202,7 +204,9 @@ __global__ __launch_bounds__(WAVE) void sink_attention_mfma_kernel(
         if (q0 + 16 * t + r >= n_new) continue;
         const size_t row = (size_t)cu_new[b] + qi[t];
         bf16_t* op = out + (row * heads + h) * vdim;
-        const bf16_t* gp = gate ? gate + row * gate_stride + (size_t)h * vdim : nullptr;
+        const bf16_t* gp = gate && !gate_per_head ? gate + row * gate_stride + (size_t)h * vdim : nullptr;
+        // one gate value for the whole head: its sigmoid goes into the factor that divides by the sum
+        const float fh = gate && gate_per_head ? f / (1.0f + __expf(-to_float(gate[row * gate_stride + h]))) : f;
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
             const int vd = 16 * vt + 4 * g;
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(WAVE) void sink_attention_mfma_kernel(
                 float o[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    o[i] = acc[t][vt][i] * f;
+                    o[i] = acc[t][vt][i] * fh;
                     if (gp) o[i] *= 1.0f / (1.0f + __expf(-to_float(gp[vd + i])));
                 }
                 uint2 w;
@@ -225,8 +229,8 @@ __global__ __launch_bounds__(WAVE) void sink_attention_mfma_kernel(
 PALM_API int palm_sink_attention_mfma(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
                                       const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                       const int* seq_new, const int* cu_new, int n_seqs, int max_new, int heads, int kv_heads,
-                                      int dim, int vdim, float scale, int window, int has_sink, float sink_score, const void* gate,
-                                      int gate_stride, void* out) {
+                                      int dim, int vdim, float scale, int window, int has_sink, float sink_score,
+                                      const float* sink_scores, const void* gate, int gate_stride, int gate_per_head, void* out) {
     PALM_CHECK(n_seqs >= 0 && max_new >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0,
                "sink_attention_mfma: seqs=%d max_new=%d heads=%d kv=%d dim=%d vdim=%d", n_seqs, max_new, heads, kv_heads, dim, vdim);
     PALM_CHECK(heads % kv_heads == 0, "sink_attention_mfma: %d heads are not a multiple of %d kv heads", heads, kv_heads);
@@ -240,7 +244,8 @@ PALM_API int palm_sink_attention_mfma(hipStream_t stream, const void* q, const v
     dim3 grid((max_new + SM_QUERIES - 1) / SM_QUERIES, heads, n_seqs);
     sink_attention_mfma_kernel<<<grid, WAVE, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, seq_slot, seq_start, seq_new,
-        cu_new, heads, kv_heads, dim, vdim, scale, window, has_sink, sink_score, (const bf16_t*)gate, gate_stride, (bf16_t*)out);
+        cu_new, heads, kv_heads, dim, vdim, scale, window, has_sink, sink_score, sink_scores, (const bf16_t*)gate, gate_stride, gate_per_head,
+        (bf16_t*)out);
     PALM_LAUNCHED();
     return 0;
 }

@@ -93,12 +93,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_place_kernel(const int* __re
 }
 
 // grid (tiles, blocks of GT_FEATURES features).  a: the rows [*, k_dim]; row_of_slot: null (the rows lie in slot order) or
-// slot -> pair, the pair's row being pair / top.  w: [experts, n_w_rows, k_dim]; GATED: n_w_rows = 2 n_features, an expert's
-// gate rows first, and the result is silu(gate) * up.  out: bfloat16 [slots, n_features].
-template <bool GATED>
+// slot -> pair, the pair's row being pair / top.  w: [experts, n_w_rows, k_dim]; FORM 1 (gated): n_w_rows = 2 n_features, an
+// expert's gate rows first, and the result is silu(gate) * up; FORM 2: the product through the exact gelu; FORM 0: the product
+// as it is.  out: bfloat16 [slots, n_features].
+template <int FORM>
 __global__ __launch_bounds__(GT_WAVES * WAVE) void moe_grouped_kernel(const bf16_t* __restrict__ a, const int* __restrict__ slot_pair, int top,
                                                                       const bf16_t* __restrict__ w, const int* __restrict__ tile_expert,
                                                                       int n_features, int k_dim, bf16_t* __restrict__ out) {
+    constexpr bool GATED = FORM == 1;
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;
@@ -154,6 +156,9 @@ __global__ __launch_bounds__(GT_WAVES * WAVE) void moe_grouped_kernel(const bf16
                 if (GATED) {
                     const float gt = acc[ft][tt][i];
                     v[i] = gt / (1.0f + expf(-gt)) * acc[2 + ft][tt][i];
+                } else if (FORM == 2) {
+                    const float z = acc[ft][tt][i];
+                    v[i] = 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
                 } else {
                     v[i] = acc[ft][tt][i];
                 }
@@ -178,12 +183,14 @@ __global__ void moe_combine_kernel(const bf16_t* __restrict__ y, const int* __re
 
 PALM_API int palm_moe_tile_tokens() { return GT_TOKENS; }
 
-// chosen, weight [n, top]; h bfloat16 [n, width]; gate_up bfloat16 [experts, 2 ff, width]; down bfloat16 [experts, width, ff].
+// chosen, weight [n, top]; h bfloat16 [n, width]; gate_up bfloat16 [experts, 2 ff, width] (form 1: [experts, ff, width], up rows
+// alone, through the exact gelu); down bfloat16 [experts, width, ff].
 // Room, with max_tiles = ceil(n top / tile) + experts and slots = max_tiles * tile: plan: (2 experts + 1 + max_tiles + slots
 // + n top) ints; mid: slots * ff bfloat16; y: slots * width bfloat16.  out float32 [n, width].
 PALM_API int palm_moe_grouped(hipStream_t stream, const void* h, const void* gate_up, const void* down, const int* chosen,
                               const float* weight, int n_tokens, int top, int experts, int width, int ff, int* plan, void* mid, void* y,
-                              float* out) {
+                              float* out, int form) {
+    PALM_CHECK(form == 0 || form == 1, "moe_grouped: form %d is neither gated silu (0) nor plain gelu (1)", form);
     PALM_CHECK(n_tokens >= 0 && top > 0 && experts > 0 && width > 0 && ff > 0, "moe_grouped: n=%d top=%d experts=%d width=%d ff=%d", n_tokens,
                top, experts, width, ff);
     PALM_CHECK(width % 8 == 0 && ff % 8 == 0, "moe_grouped: width %d and inner size %d must be multiples of eight", width, ff);
@@ -199,9 +206,13 @@ PALM_API int palm_moe_grouped(hipStream_t stream, const void* h, const void* gat
     moe_count_kernel<<<experts, PLAN_THREADS, 0, stream>>>(chosen, (int)n_pairs, counts);
     moe_runs_kernel<<<1, PLAN_THREADS, 0, stream>>>(counts, experts, max_tiles, starts, tile_expert);
     moe_place_kernel<<<experts, PLAN_THREADS, 0, stream>>>(chosen, (int)n_pairs, starts, slot_pair, pair_slot);
-    moe_grouped_kernel<true><<<dim3(max_tiles, (ff + GT_FEATURES - 1) / GT_FEATURES), GT_WAVES * WAVE, 0, stream>>>(
-        (const bf16_t*)h, slot_pair, top, (const bf16_t*)gate_up, tile_expert, ff, width, (bf16_t*)mid);
-    moe_grouped_kernel<false><<<dim3(max_tiles, (width + GT_FEATURES - 1) / GT_FEATURES), GT_WAVES * WAVE, 0, stream>>>(
+    if (form == 0)
+        moe_grouped_kernel<1><<<dim3(max_tiles, (ff + GT_FEATURES - 1) / GT_FEATURES), GT_WAVES * WAVE, 0, stream>>>(
+            (const bf16_t*)h, slot_pair, top, (const bf16_t*)gate_up, tile_expert, ff, width, (bf16_t*)mid);
+    else
+        moe_grouped_kernel<2><<<dim3(max_tiles, (ff + GT_FEATURES - 1) / GT_FEATURES), GT_WAVES * WAVE, 0, stream>>>(
+            (const bf16_t*)h, slot_pair, top, (const bf16_t*)gate_up, tile_expert, ff, width, (bf16_t*)mid);
+    moe_grouped_kernel<0><<<dim3(max_tiles, (width + GT_FEATURES - 1) / GT_FEATURES), GT_WAVES * WAVE, 0, stream>>>(
         (const bf16_t*)mid, nullptr, top, (const bf16_t*)down, tile_expert, width, ff, (bf16_t*)y);
     moe_combine_kernel<<<n_tokens, 256, 0, stream>>>((const bf16_t*)y, pair_slot, weight, top, width, out);
     PALM_LAUNCHED();

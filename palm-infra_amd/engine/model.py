@@ -9,7 +9,8 @@ from __future__ import annotations
 import torch
 
 from ..config.spec import ModelSpec
-from ..parts import Builder, ResidualSink, cache_needs
+from ..kernels import ops
+from ..parts import Builder, ResidualSink, cache_needs, cache_needs_beside_shared
 
 
 class DecoderModel:
@@ -38,7 +39,8 @@ class DecoderModel:
                 needs.append(cache_needs(self.spec.layers[call.layer]))
                 shares.append(None)
             else:
-                needs.append([])
+                # what the entry keeps of its own beside the storage that it reads (a state of its own projections)
+                needs.append(cache_needs_beside_shared(self.spec.layers[call.layer]))
                 shares.append(call.cache_of)
         return needs, shares
 
@@ -52,6 +54,8 @@ class DecoderModel:
             x = self.embedding.forward(ctx.token_ids, out=ctx.results[0]).clone()
         else:
             x = self.embedding.forward(ctx.token_ids)
+        if self.spec.streams is not None and self.spec.streams > 1:
+            x = ops.streams_spread(x, self.spec.streams)        # every copy starts as the embedding's rows
         if not self.order:
             return self.head.forward(self.final_norm(x, rows=want_rows))
         # a layer gets its first norm's output and returns the output of the norm after it: the next layer's

@@ -17,8 +17,11 @@ Libraries:
   ``branches``          branch outputs scaled by a learned vector into the residual stream; the capped feed-forward gate
   ``mixers``            the other mixers beside softmax attention over equal key and value sizes (the selective
                         scan and its convolution, differential attention, the delta rule, attention over compressed
-                        rows), routed experts, and the stream of blocks that norm a branch's output; loaded when a
-                        model has such a part
+                        rows), and the stream of blocks that norm a branch's output; loaded when a model has such a part
+  ``feedforward``       routed experts (routing by softmax or by scores in groups, experts gated or plain) and the
+                        activations of plain feed-forwards
+  ``streams``           a residual stream in several copies with learned weights between them, and its norms
+  ``mlstm``             a matrix memory with input and forget gates per head and token
   ``latent_attention_k<K>_v<V>``  attention over compressed rows for prompts on the matrix cores, compiled for rows up to
                         32 K and latents up to 16 V
   ``attention_diff_k<K>_v<V>_q<Q>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
@@ -56,7 +59,10 @@ ATTENTION_SOURCES = ["attention_mfma.hip"]
 DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
 LATENT_ATTENTION_SOURCES = ["latent_attention_mfma.hip"]
 MIXER_SOURCES = ["stream.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
-                 "latent_attention.hip", "moe.hip", "moe_grouped.hip"]
+                 "latent_attention.hip"]
+FEEDFORWARD_SOURCES = ["moe.hip", "moe_grouped.hip", "activation.hip"]
+STREAMS_SOURCES = ["streams.hip"]
+MLSTM_SOURCES = ["mlstm.hip"]
 RECURRENT_SOURCES = ["retention.hip"]
 SINK_ATTENTION_SOURCES = ["attention_sink.hip"]
 SINK_ATTENTION_MFMA_SOURCES = ["attention_sink_mfma.hip"]
@@ -199,6 +205,12 @@ def _spec(name: str):
         return SINK_ATTENTION_SOURCES, ()
     if name == "branches":
         return BRANCH_SOURCES, ()
+    if name == "feedforward":
+        return FEEDFORWARD_SOURCES, ()
+    if name == "streams":
+        return STREAMS_SOURCES, ()
+    if name == "mlstm":
+        return MLSTM_SOURCES, ()
     if name.startswith("sink_attention_k"):
         kk, vt = name[len("sink_attention_k"):].split("_v")
         return SINK_ATTENTION_MFMA_SOURCES, (f"PALM_SINK_KK={int(kk)}", f"PALM_SINK_VT={int(vt)}")

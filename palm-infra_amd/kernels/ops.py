@@ -784,14 +784,6 @@ _MIXER_SIGNATURES = {
     "palm_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "palm_latent_output": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "palm_moe_route": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
-    "palm_moe_experts": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                         c_void_p, c_void_p],
-    "palm_moe_tile_tokens": [],
-    "palm_moe_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
-                         c_void_p, c_void_p],
-    "palm_gather_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "palm_scatter_add": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 _mixers = None
 
@@ -818,10 +810,34 @@ _RECURRENT_SIGNATURES = {
 _SINK_SIGNATURES = {
     "palm_sink_qkv_store": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                             c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                            c_int, c_int, c_int],
+                            c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     "palm_sink_attention": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_int, c_int,
-                            c_void_p, c_void_p],
+                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_void_p, c_int,
+                            c_int, c_int, c_void_p, c_void_p],
+}
+_FEEDFORWARD_SIGNATURES = {
+    "palm_moe_route": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+    "palm_moe_route_scored": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p],
+    "palm_add_gated_rows": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int],
+    "palm_moe_experts": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_void_p, c_void_p, c_int],
+    "palm_moe_tile_tokens": [],
+    "palm_moe_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                         c_void_p, c_void_p, c_int],
+    "palm_gather_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "palm_scatter_add": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "palm_activation": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_longlong],
+}
+_STREAMS_SIGNATURES = {
+    "palm_streams_spread": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "palm_streams_mix_norm": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                              c_void_p, c_float, c_float, c_void_p, c_int, c_int, c_void_p, c_int],
+}
+_MLSTM_SIGNATURES = {
+    "palm_mlstm_pad": [c_int],
+    "palm_mlstm": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_float,
+                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                   c_int, c_void_p, c_void_p],
 }
 _BRANCH_SIGNATURES = {
     "palm_add_scaled_normed": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_int, c_void_p, c_void_p, c_float, c_void_p,
@@ -853,6 +869,18 @@ def sink_attention_lib():
 
 def branches():
     return _small("branches", _BRANCH_SIGNATURES)
+
+
+def feedforward():
+    return _small("feedforward", _FEEDFORWARD_SIGNATURES)
+
+
+def streams_lib():
+    return _small("streams", _STREAMS_SIGNATURES)
+
+
+def mlstm_lib():
+    return _small("mlstm", _MLSTM_SIGNATURES)
 
 
 def add_normed(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
@@ -1370,25 +1398,79 @@ def moe_route(logits: torch.Tensor, top: int):
     n, experts = logits.shape
     chosen = torch.empty((n, top), dtype=torch.int32, device=logits.device)
     weight = torch.empty((n, top), dtype=F32, device=logits.device)
-    library.call(mixers(), "palm_moe_route", _stream(), _p(logits), n, experts, int(top), _p(chosen), _p(weight))
+    library.call(feedforward(), "palm_moe_route", _stream(), _p(logits), n, experts, int(top), _p(chosen), _p(weight))
     return chosen, weight
 
 
-def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int) -> torch.Tensor:
+EXPERT_FORMS = {"gated_silu": 0, "gelu": 1}
+
+
+def _expert_shapes(what, h, up, down, ff, form):
+    """-> (experts, rows of an expert's first matrix): gated experts keep their gate rows before their up rows."""
+    _need(form in EXPERT_FORMS, f"{what}: an expert's form {form!r} is not one of {sorted(EXPERT_FORMS)}")
+    per = (2 if form == "gated_silu" else 1) * ff
+    width = h.shape[1]
+    _need(up.dim() == 2 and up.shape[1] == width and up.shape[0] % per == 0 and down.shape == (up.shape[0] // per * width, ff)
+          and up.dtype == down.dtype, f"{what}: first matrices {tuple(up.shape)}, down {tuple(down.shape)} for width {width}, inner size {ff}")
+    return up.shape[0] // per
+
+
+def moe_route_scored(logits: torch.Tensor, experts: int, top: int, correction: torch.Tensor | None, groups: int, keep: int, scale: float):
+    """logits float32 [n, >= experts] (the experts' columns first) -> (chosen int32 [n, top], weight float32 [n, top]).  The
+    scores are sigmoid(logit); the choice is made by score + ``correction``; the experts lie in ``groups`` equal groups of
+    neighbours, a group ranks by the sum of its two largest corrected scores, and only experts of the best ``keep`` groups can
+    be chosen (the lower index wins a tie); the weights are the chosen scores over their sum (+ 1e-20), times ``scale``."""
+    _dev("moe_route_scored", logits, correction)
+    _need(logits.dim() == 2 and logits.dtype == F32 and logits.shape[1] >= experts, f"moe_route_scored: router logits are float32 [n, >= {experts}], "
+          f"not {logits.dtype} {tuple(logits.shape)}")
+    _need(correction is None or (correction.shape == (experts,) and correction.dtype == F32), f"moe_route_scored: the correction is float32 [{experts}]")
+    n = logits.shape[0]
+    chosen = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((n, top), dtype=F32, device=logits.device)
+    library.call(feedforward(), "palm_moe_route_scored", _stream(), _p(logits), logits.shape[1], n, int(experts), int(top), _p(correction),
+                 int(groups), int(keep), float(scale), _p(chosen), _p(weight))
+    return chosen, weight
+
+
+def add_gated_rows(out: torch.Tensor, y: torch.Tensor, logits: torch.Tensor, column: int) -> torch.Tensor:
+    """out[t] += sigmoid(logits[t, column]) * y[t]: out float32 [n, width] in place, logits float32 [n, *]."""
+    _dev("add_gated_rows", out, y, logits)
+    _need(out.dim() == 2 and out.dtype == F32 and y.shape == out.shape and logits.dim() == 2 and logits.dtype == F32
+          and logits.shape[0] == out.shape[0] and 0 <= column < logits.shape[1],
+          f"add_gated_rows: out {tuple(out.shape)} {out.dtype}, y {tuple(y.shape)}, gate column {column} of {tuple(logits.shape)} {logits.dtype}")
+    library.call(feedforward(), "palm_add_gated_rows", _stream(), _p(out), _p(y), _code(y, "add_gated_rows"),
+                 logits.data_ptr() + column * 4, logits.shape[1], out.shape[0], out.shape[1])
+    return out
+
+
+ACTIVATIONS = {"relu_squared": 0, "gelu_erf": 1, "gelu_tanh": 2}
+
+
+def activation(z: torch.Tensor, kind: str) -> torch.Tensor:
+    """max(z, 0)^2, or the gelu with erf, or the gelu with tanh, elementwise, 32-bit inside."""
+    _dev("activation", z)
+    _need(kind in ACTIVATIONS, f"activation: {kind!r} is not one of {sorted(ACTIVATIONS)}")
+    out = torch.empty_like(z)
+    library.call(feedforward(), "palm_activation", _stream(), _p(z), _p(out), _code(z, "activation"), ACTIVATIONS[kind], z.numel())
+    return out
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int,
+                form: str = "gated_silu") -> torch.Tensor:
     """Every row through its chosen experts, nothing planned on the host: h [n, width]; gate_up [experts * 2 ff, width] (an
-    expert's gate rows, then its up rows); down [experts * width, ff].  Returns float32 [n, width], the weighted sum."""
+    expert's gate rows, then its up rows; ``form`` "gelu": [experts * ff, width], up rows alone, through the exact gelu);
+    down [experts * width, ff].  Returns float32 [n, width], the weighted sum."""
     what = "moe_experts"
     _dev(what, h, gate_up, down, chosen, weight)
     _i32(what, chosen)
     n, width = h.shape
     top = chosen.shape[1]
-    _need(gate_up.dim() == 2 and gate_up.shape[1] == width and gate_up.shape[0] % (2 * ff) == 0 and down.shape == (gate_up.shape[0] // (2 * ff) * width, ff)
-          and gate_up.dtype == down.dtype, f"{what}: gate/up {tuple(gate_up.shape)}, down {tuple(down.shape)} for width {width}, inner size {ff}")
+    _expert_shapes(what, h, gate_up, down, ff, form)
     _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == F32, f"{what}: choices {tuple(chosen.shape)}, weights {tuple(weight.shape)}")
     mid = torch.empty((n, top, ff), dtype=F32, device=h.device)
     out = torch.empty((n, width), dtype=F32, device=h.device)
-    library.call(mixers(), "palm_moe_experts", _stream(), _p(h), _code(h, what), _p(gate_up), _p(down), _code(gate_up, what + " weights"),
-                 _p(chosen), _p(weight), n, top, width, ff, _p(mid), _p(out))
+    library.call(feedforward(), "palm_moe_experts", _stream(), _p(h), _code(h, what), _p(gate_up), _p(down), _code(gate_up, what + " weights"),
+                 _p(chosen), _p(weight), n, top, width, ff, _p(mid), _p(out), EXPERT_FORMS[form])
     return out
 
 
@@ -1397,7 +1479,8 @@ def moe_grouped_serves(h: torch.Tensor, gate_up: torch.Tensor, ff: int) -> bool:
     return h.dtype == BF16 and gate_up.dtype == BF16 and h.shape[1] % 8 == 0 and ff % 8 == 0
 
 
-def moe_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int) -> torch.Tensor:
+def moe_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int,
+                form: str = "gated_silu") -> torch.Tensor:
     """Every row through its chosen experts, for many rows, planned on the device: the (row, choice) pairs grouped by expert,
     two grouped products on the matrix cores, the weighted sum in the order of the choices.  Shapes as ``moe_experts``;
     returns float32 [n, width]."""
@@ -1407,19 +1490,18 @@ def moe_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chos
     n, width = h.shape
     top = chosen.shape[1]
     _need(moe_grouped_serves(h, gate_up, ff), f"{what}: bfloat16 rows and weights, sizes in multiples of eight")
-    _need(gate_up.dim() == 2 and gate_up.shape[1] == width and gate_up.shape[0] % (2 * ff) == 0 and down.shape == (gate_up.shape[0] // (2 * ff) * width, ff)
-          and down.dtype == BF16, f"{what}: gate/up {tuple(gate_up.shape)}, down {tuple(down.shape)} for width {width}, inner size {ff}")
+    experts = _expert_shapes(what, h, gate_up, down, ff, form)
+    _need(down.dtype == BF16, f"{what}: bfloat16 weights")
     _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == F32, f"{what}: choices {tuple(chosen.shape)}, weights {tuple(weight.shape)}")
-    experts = gate_up.shape[0] // (2 * ff)
-    tile = mixers().palm_moe_tile_tokens()
+    tile = feedforward().palm_moe_tile_tokens()
     max_tiles = (n * top + tile - 1) // tile + experts
     slots = max_tiles * tile
     plan = torch.empty((2 * experts + 1 + max_tiles + slots + n * top,), dtype=torch.int32, device=h.device)
     mid = torch.empty((slots, ff), dtype=BF16, device=h.device)
     y = torch.empty((slots, width), dtype=BF16, device=h.device)
     out = torch.empty((n, width), dtype=F32, device=h.device)
-    library.call(mixers(), "palm_moe_grouped", _stream(), _p(h), _p(gate_up), _p(down), _p(chosen), _p(weight), n, top, experts, width, ff,
-                 _p(plan), _p(mid), _p(y), _p(out))
+    library.call(feedforward(), "palm_moe_grouped", _stream(), _p(h), _p(gate_up), _p(down), _p(chosen), _p(weight), n, top, experts, width, ff,
+                 _p(plan), _p(mid), _p(y), _p(out), EXPERT_FORMS[form])
     return out
 
 
@@ -1429,7 +1511,7 @@ def gather_rows(h: torch.Tensor, src: torch.Tensor) -> torch.Tensor:
     _i32("gather_rows", src)
     _need(h.dim() == 2 and src.dim() == 1, f"gather_rows: rows {tuple(h.shape)}, indices {tuple(src.shape)}")
     xs = torch.empty((src.shape[0], h.shape[1]), dtype=h.dtype, device=h.device)
-    library.call(mixers(), "palm_gather_rows", _stream(), _p(h), _code(h, "gather_rows"), _p(src), src.shape[0], h.shape[1], _p(xs))
+    library.call(feedforward(), "palm_gather_rows", _stream(), _p(h), _code(h, "gather_rows"), _p(src), src.shape[0], h.shape[1], _p(xs))
     return xs
 
 
@@ -1440,7 +1522,7 @@ def scatter_add(out: torch.Tensor, y: torch.Tensor, rows: torch.Tensor, weight: 
     _need(out.dtype == F32 and out.dim() == 2 and y.dim() == 2 and y.shape[1] == out.shape[1] and rows.shape == (y.shape[0],)
           and weight.shape == (y.shape[0],) and weight.dtype == F32, f"scatter_add: out {tuple(out.shape)} {out.dtype}, y {tuple(y.shape)}, "
           f"rows {tuple(rows.shape)}, weights {tuple(weight.shape)} {weight.dtype}")
-    library.call(mixers(), "palm_scatter_add", _stream(), _p(y), _code(y, "scatter_add"), _p(rows), _p(weight), y.shape[0], out.shape[1], _p(out))
+    library.call(feedforward(), "palm_scatter_add", _stream(), _p(y), _code(y, "scatter_add"), _p(rows), _p(weight), y.shape[0], out.shape[1], _p(out))
 
 
 # ---- softmax attention with a sink, a window and a gate (library ``sink_attention``) -------------------------------
@@ -1449,37 +1531,65 @@ SINK_NORMS = {None: 0, "projection": 1, "head": 2}
 SINK_BLOCKS_WANTED = 1024         # a decode step's key ranges are cut into slices until about this many blocks run
 
 
+ROTARY_PAIRINGS = {"half_split": 0, "interleaved": 1}
+
+
 def sink_qkv_store(rows: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, bias, norm: str | None, q_w, k_w, eps: float,
-                   cos, sin, rot: int, k_cache, v_cache, block_table, ctx, write_cache: bool = True, col0: int = 0) -> torch.Tensor:
+                   cos, sin, rot: int, k_cache, v_cache, block_table, ctx, write_cache: bool = True, col0: int = 0,
+                   pairing: str = "half_split", conv=None, conv_state=None) -> torch.Tensor:
     """q, k and v of the step's tokens from ``rows`` [n, >= heads*dim + kv_heads*dim + kv_heads*vdim] (q | k | v | whatever
     follows): ``bias`` (float32 over q | k | v, or None) is added, q and k are normed (``norm``: "projection": one RMS norm
     over the whole q row and one over the whole k row, weights of those sizes; "head": per head, weights of the key size;
-    None), their first ``rot`` dimensions are rotated by the tokens' cos and sin rows, k and v go to their pages, and q
-    comes back as [n, heads, dim].  ``col0``: q begins at this column of the rows."""
-    _dev("sink_qkv_store", rows, bias, q_w, k_w, cos, sin, k_cache, v_cache, block_table, ctx.tok_slot, ctx.positions)
+    None), their first ``rot`` dimensions are rotated by the tokens' cos and sin rows (``pairing``: dimension i with i + rot/2,
+    or 2i with 2i + 1), k and v go to their pages, and q comes back as [n, heads, dim].  ``col0``: q begins at this column of
+    the rows.
+
+    ``write_cache`` false: the layer reads another layer's keys and values; the rows hold q alone (| whatever follows) and
+    bias, convolution and state cover q's channels only.
+
+    ``conv`` (float32 [channels, taps], q | k | v) with ``conv_state`` (float32 [slots, taps - 1, channels]): right after
+    the bias every channel goes through a short causal convolution over time, y_t = sum_j conv[c, j] u_(t - taps + 1 + j);
+    the state holds each sequence's last taps - 1 inputs (zero for a new sequence) and is left updated."""
+    _dev("sink_qkv_store", rows, bias, q_w, k_w, cos, sin, block_table, ctx.tok_slot, ctx.positions, conv, conv_state)
     _i32("sink_qkv_store", block_table, ctx.tok_slot, ctx.positions)
     n = rows.shape[0]
-    q_size, k_size, v_size = heads * dim, kv_heads * dim, kv_heads * vdim
-    _need(rows.dim() == 2 and col0 >= 0 and rows.shape[1] >= col0 + q_size + k_size + v_size and n == ctx.n_tokens,
+    q_size = heads * dim
+    k_size, v_size = (kv_heads * dim, kv_heads * vdim) if write_cache else (0, 0)
+    channels = q_size + k_size + v_size
+    _need(rows.dim() == 2 and col0 >= 0 and rows.shape[1] >= col0 + channels and n == ctx.n_tokens,
           f"sink_qkv_store: rows {tuple(rows.shape)} for {ctx.n_tokens} tokens of {q_size} + {k_size} + {v_size}")
     _need(norm in SINK_NORMS, f"sink_qkv_store: norm {norm!r} is not one of {sorted(map(str, SINK_NORMS))}")
+    _need(pairing in ROTARY_PAIRINGS, f"sink_qkv_store: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     if bias is not None:
-        _need(bias.shape == (q_size + k_size + v_size,) and bias.dtype == F32, f"sink_qkv_store: the bias is float32 [{q_size + k_size + v_size}]")
+        _need(bias.shape == (channels,) and bias.dtype == F32, f"sink_qkv_store: the bias is float32 [{channels}]")
     if norm is not None:
-        want = (q_size, k_size) if norm == "projection" else (dim, dim)
+        want = (q_size, kv_heads * dim) if norm == "projection" else (dim, dim)
         _need(q_w is not None and k_w is not None and q_w.shape == (want[0],) and k_w.shape == (want[1],) and q_w.dtype == F32
               and k_w.dtype == F32, f"sink_qkv_store: the norm weights are float32 [{want[0]}] and [{want[1]}]")
     if rot:
         for tab in (cos, sin):
             _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"sink_qkv_store: rotation rows are float32 [{n}, {rot // 2}]")
-    _need(k_cache.dtype == rows.dtype and v_cache.dtype == rows.dtype and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
-          and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS) and block_table.dim() == 2,
-          f"sink_qkv_store: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} for rows of {rows.dtype}")
+    if write_cache:
+        _dev("sink_qkv_store", k_cache, v_cache)
+        _need(k_cache.dtype == rows.dtype and v_cache.dtype == rows.dtype and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
+              and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS) and block_table.dim() == 2,
+              f"sink_qkv_store: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} for rows of {rows.dtype}")
+    taps = 0
+    if conv is not None:
+        taps = conv.shape[1] if conv.dim() == 2 else -1
+        _need(conv.shape == (channels, taps) and conv.dtype == F32 and taps >= 1, f"sink_qkv_store: the convolution is float32 [{channels}, taps], not {tuple(conv.shape)}")
+        if taps > 1:
+            _need(conv_state is not None and conv_state.dim() == 3 and conv_state.shape[1:] == (taps - 1, channels) and conv_state.dtype == F32,
+                  f"sink_qkv_store: the convolution's state is float32 [slots, {taps - 1}, {channels}]")
+            _dev("sink_qkv_store", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+            _i32("sink_qkv_store", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     q = torch.empty((n, heads, dim), dtype=rows.dtype, device=rows.device)
     library.call(sink_attention_lib(), "palm_sink_qkv_store", _stream(), _p(rows), _code(rows, "sink_qkv_store"), rows.shape[1], col0, col0 + q_size,
-                 col0 + q_size + k_size, _p(bias), _p(q), _p(k_cache), _p(v_cache), _p(block_table), block_table.shape[1], _p(ctx.tok_slot),
+                 col0 + q_size + k_size, _p(bias), _p(q), _p(k_cache) if write_cache else None, _p(v_cache) if write_cache else None,
+                 _p(block_table), block_table.shape[1], _p(ctx.tok_slot),
                  _p(ctx.positions), SINK_NORMS[norm], _p(q_w), _p(k_w), float(eps), _p(cos), _p(sin), int(rot), n, heads, kv_heads, dim,
-                 vdim, int(write_cache))
+                 vdim, int(write_cache), ROTARY_PAIRINGS[pairing], _p(conv), int(taps), _p(conv_state) if taps > 1 else None,
+                 _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs)
     return q
 
 
@@ -1496,11 +1606,12 @@ def sink_slices(ctx, heads: int, kv_heads: int, window: int | None) -> int:
 
 
 def sink_attention_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
-                         scale: float, window: int | None, sink: float | None, gate: torch.Tensor | None, gate_off: int = 0,
-                         slices: int | None = None) -> torch.Tensor:
+                         scale: float, window: int | None, sink, gate: torch.Tensor | None, gate_off: int = 0,
+                         slices: int | None = None, gate_per_head: bool = False) -> torch.Tensor:
     """Attention of the step's queries q [n, heads, dim] over the cached keys of their sequences up to their own positions
-    (the last ``window`` if given), with a sink of score ``sink`` (None: none) in the denominator.  ``gate``: a tensor [n,
-    >= gate_off + heads*vdim] whose columns from ``gate_off`` on gate the output through a sigmoid (None: no gate).  Returns
+    (the last ``window`` if given), with a sink in the denominator: ``sink`` is its score for all heads, or a float32 tensor
+    [heads] of learned scores, or None.  ``gate``: a tensor [n, >= gate_off + heads*vdim] whose columns from ``gate_off`` on
+    gate the output through a sigmoid (None: no gate); with ``gate_per_head`` one column for each head.  Returns
     [n, heads * vdim].  32-bit arithmetic whatever the elements' type."""
     _dev("sink_attention", q, k_cache, v_cache, block_table, gate, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
     _i32("sink_attention", block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
@@ -1508,23 +1619,39 @@ def sink_attention_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, he
     _need(q.shape == (ctx.n_tokens, heads, dim), f"sink_attention: q {tuple(q.shape)} is not [{ctx.n_tokens}, {heads}, {dim}]")
     _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
           and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS), f"sink_attention: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
-    gate_ptr, gate_stride = None, 0
-    if gate is not None:
-        _need(gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= gate_off + heads * vdim and gate.dtype == q.dtype,
-              f"sink_attention: gate rows {tuple(gate.shape)} {gate.dtype} from column {gate_off}")
-        gate_ptr, gate_stride = gate.data_ptr() + gate_off * gate.element_size(), gate.shape[1]
+    gate_ptr, gate_stride = _sink_gate("sink_attention", gate, gate_off, n, heads, vdim, q.dtype, gate_per_head)
+    sink_score, sink_scores = _sink_scores("sink_attention", sink, heads, q.device)
     slices = sink_slices(ctx, heads, kv_heads, window) if slices is None else int(slices)
     work = torch.empty((n * heads * slices * (vdim + 2),), dtype=F32, device=q.device) if slices > 1 else None
     out = torch.empty((n, heads * vdim), dtype=q.dtype, device=q.device)
     library.call(sink_attention_lib(), "palm_sink_attention", _stream(), _p(q), _code(q, "sink_attention"), _p(k_cache), _p(v_cache),
                  _p(block_table), block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs,
                  int(ctx.max_new), n, heads, kv_heads, dim, vdim, float(scale), int(window or 0), int(sink is not None),
-                 float(sink or 0.0), gate_ptr, gate_stride, slices, _p(work), _p(out))
+                 sink_score, _p(sink_scores), gate_ptr, gate_stride, int(gate_per_head), slices, _p(work), _p(out))
     return out
 
 
+def _sink_gate(what: str, gate, gate_off: int, n: int, heads: int, vdim: int, dtype, per_head: bool):
+    """(address of token 0's first gate value, elements between rows), or (None, 0)."""
+    if gate is None:
+        return None, 0
+    cols = heads if per_head else heads * vdim
+    _need(gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= gate_off + cols and gate.dtype == dtype,
+          f"{what}: gate rows {tuple(gate.shape)} {gate.dtype} with {cols} columns from column {gate_off}")
+    return gate.data_ptr() + gate_off * gate.element_size(), gate.shape[1]
+
+
+def _sink_scores(what: str, sink, heads: int, device):
+    """(one score for all heads, a tensor of one for each or None)."""
+    if isinstance(sink, torch.Tensor):
+        _dev(what, sink)
+        _need(sink.shape == (heads,) and sink.dtype == F32, f"{what}: learned sink scores are float32 [{heads}], not {sink.dtype} {tuple(sink.shape)}")
+        return 0.0, sink
+    return float(sink or 0.0), None
+
+
 _SINK_MFMA_SIGNATURE = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_int, c_void_p]
+                        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p]
 _sink_mfma_libs: dict = {}
 
 
@@ -1545,7 +1672,8 @@ def sink_attention_mfma_lib(dim: int, vdim: int):
 
 
 def sink_attention_mfma(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
-                        scale: float, window: int | None, sink: float | None, gate: torch.Tensor | None, gate_off: int = 0) -> torch.Tensor:
+                        scale: float, window: int | None, sink, gate: torch.Tensor | None, gate_off: int = 0,
+                        gate_per_head: bool = False) -> torch.Tensor:
     """``sink_attention_exact`` for prompts in bfloat16 on the matrix cores (scores, weights and sums 32-bit)."""
     _dev("sink_attention_mfma", q, k_cache, v_cache, block_table, gate, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
     _i32("sink_attention_mfma", block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
@@ -1554,25 +1682,25 @@ def sink_attention_mfma(q: torch.Tensor, k_cache, v_cache, block_table, ctx, hea
     _need(q.shape == (ctx.n_tokens, heads, dim), f"sink_attention_mfma: q {tuple(q.shape)} is not [{ctx.n_tokens}, {heads}, {dim}]")
     _need(k_cache.dtype == BF16 and v_cache.dtype == BF16 and k_cache.shape[1:] == (kv_heads, PAGE_TOKENS, dim)
           and v_cache.shape[1:] == (kv_heads, vdim, PAGE_TOKENS), f"sink_attention_mfma: cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
-    gate_ptr, gate_stride = None, 0
-    if gate is not None:
-        _need(gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= gate_off + heads * vdim and gate.dtype == BF16,
-              f"sink_attention_mfma: gate rows {tuple(gate.shape)} {gate.dtype} from column {gate_off}")
-        gate_ptr, gate_stride = gate.data_ptr() + gate_off * gate.element_size(), gate.shape[1]
+    gate_ptr, gate_stride = _sink_gate("sink_attention_mfma", gate, gate_off, n, heads, vdim, BF16, gate_per_head)
+    sink_score, sink_scores = _sink_scores("sink_attention_mfma", sink, heads, q.device)
     out = torch.empty((n, heads * vdim), dtype=BF16, device=q.device)
     library.call(sink_attention_mfma_lib(dim, vdim), "palm_sink_attention_mfma", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
                  block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
-                 heads, kv_heads, dim, vdim, float(scale), int(window or 0), int(sink is not None), float(sink or 0.0), gate_ptr,
-                 gate_stride, _p(out))
+                 heads, kv_heads, dim, vdim, float(scale), int(window or 0), int(sink is not None), sink_score, _p(sink_scores), gate_ptr,
+                 gate_stride, int(gate_per_head), _p(out))
     return out
 
 
-def sink_attention(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off=0):
+def sink_attention(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off=0,
+                   gate_per_head=False):
     """The kernel that serves: the matrix cores for prompts in bfloat16, the exact one for the float32 mode, for single
     tokens, and for sizes that the matrix-core kernel does not take."""
     if not ctx.is_decode and sink_mfma_serves(q, dim, vdim):
-        return sink_attention_mfma(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off)
-    return sink_attention_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off)
+        return sink_attention_mfma(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off,
+                                   gate_per_head=gate_per_head)
+    return sink_attention_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, window, sink, gate, gate_off,
+                                gate_per_head=gate_per_head)
 
 
 # ---- branches scaled by a learned vector; the capped feed-forward gate (library ``branches``) ---------------------
@@ -1609,4 +1737,108 @@ def capped_gate(gate_up: torch.Tensor, limit: float, slope: float, shift: float)
     out = torch.empty((n, ff), dtype=gate_up.dtype, device=gate_up.device)
     library.call(branches(), "palm_capped_gate", _stream(), _p(gate_up), _p(out), _code(gate_up, "capped_gate"), n, ff, float(limit),
                  float(slope), float(shift))
+    return out
+
+
+# ---- a residual stream in several copies, and its norms (library ``streams``) ------------------------------------
+
+STREAM_NORMS = {None: 0, "dyt": 1, "rms": 2}
+
+
+def streams_spread(x: torch.Tensor, streams: int) -> torch.Tensor:
+    """x float32 [n, width] -> [n, streams, width]: every stream starts as a copy of x."""
+    _dev("streams_spread", x)
+    _need(x.dim() == 2 and x.dtype == F32 and streams >= 1, f"streams_spread: x {tuple(x.shape)} {x.dtype}, {streams} streams")
+    xs = torch.empty((x.shape[0], streams, x.shape[1]), dtype=F32, device=x.device)
+    library.call(streams_lib(), "palm_streams_spread", _stream(), _p(x), x.shape[0], int(streams), x.shape[1], _p(xs))
+    return xs
+
+
+def streams_mix_norm(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, out_w: torch.Tensor | None,
+                     in_w: torch.Tensor | None, norm: str | None, norm_w=None, norm_b=None, alpha: float = 1.0, eps: float = 0.0,
+                     rows: torch.Tensor | None = None, out_dtype: torch.dtype | None = None, read: bool = True):
+    """One sublayer's write into the streams and the next reader's read, in one pass.  xs float32 [n, S, width].
+
+    Write (``y`` [n, width] given): xs'[t] = sum_s mix[s, t] xs[s] + out_w[t] y, all streams at once, in place; with
+    ``rows`` the stream stays as it is and only those rows are computed, for the reader.
+    Read (``read``): u = sum_s in_w[s] xs'[s] (``in_w`` None: the plain sum), through ``norm``: "dyt" tanh(alpha u) w + b,
+    "rms" u / sqrt(mean(u^2) + eps) w, None u itself; returned in ``out_dtype`` as [rows or n, width]."""
+    what = "streams_mix_norm"
+    _dev(what, xs, y, mix, out_w, in_w, norm_w, norm_b, rows)
+    _i32(what, rows)
+    _need(xs.dim() == 3 and xs.dtype == F32, f"{what}: the streams are float32 [n, S, width], not {xs.dtype} {tuple(xs.shape)}")
+    n, S, width = xs.shape
+    _need(norm in STREAM_NORMS, f"{what}: norm {norm!r} is not one of {sorted(map(str, STREAM_NORMS))}")
+    if y is not None:
+        _need(y.shape == (n, width) and mix is not None and mix.shape == (S, S) and mix.dtype == F32 and out_w is not None
+              and out_w.shape == (S,) and out_w.dtype == F32, f"{what}: output {tuple(y.shape)} with weights {None if mix is None else tuple(mix.shape)}, "
+              f"{None if out_w is None else tuple(out_w.shape)} for {S} streams of width {width}")
+    _need(in_w is None or (in_w.shape == (S,) and in_w.dtype == F32), f"{what}: the reader's weights are float32 [{S}]")
+    _need(y is not None or read, f"{what}: neither a write nor a read")
+    out = None
+    n_rows = n if rows is None else rows.shape[0]
+    if read:
+        if norm is not None:
+            _need(norm_w is not None and norm_w.shape == (width,) and norm_w.dtype == F32 and (norm_b is None or (norm_b.shape == (width,) and norm_b.dtype == F32)),
+                  f"{what}: the norm's vectors are float32 [{width}]")
+        out = torch.empty((n_rows, width), dtype=out_dtype or F32, device=xs.device)
+    library.call(streams_lib(), "palm_streams_mix_norm", _stream(), _p(xs), n, S, width, _p(y), _code(y, what) if y is not None else 0, _p(mix),
+                 _p(out_w), _p(in_w), STREAM_NORMS[norm], _p(norm_w), _p(norm_b), float(alpha), float(eps), _p(rows), n_rows,
+                 int(rows is None and y is not None), _p(out), _code(out, what + " out") if out is not None else 0)
+    return out
+
+
+# ---- a matrix memory with gates per head and token (library ``mlstm``) ----------------------------------------------
+
+MLSTM_BLOCKS_WANTED = 512          # a long run of new tokens is cut into chunks until about this many blocks run
+MLSTM_MIN_CHUNK = 32
+
+
+def mlstm_chunk(n_seqs: int, heads: int, max_new: int) -> int:
+    """Into chunks of how many tokens the kernel cuts the step's runs of new tokens (0: not at all): where one block per
+    (head, sequence) leaves most of the chip idle and the runs are long, chunks run side by side at the price of walking
+    over every token twice."""
+    per_seq = MLSTM_BLOCKS_WANTED // max(1, heads * n_seqs)
+    if max_new <= 2 * MLSTM_MIN_CHUNK or per_seq <= 1:
+        return 0
+    chunk = max(MLSTM_MIN_CHUNK, -(-max_new // per_seq))
+    chunk = (chunk + 7) // 8 * 8
+    return chunk if chunk < max_new else 0
+
+
+def mlstm(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor | None, heads: int, dim: int, vdim: int, cap: float,
+          q_scale: float, norm_w: torch.Tensor, eps: float, state: torch.Tensor, m_state: torch.Tensor, ctx, col0: int = 0,
+          chunk: int | None = None) -> torch.Tensor:
+    """The step's tokens through a matrix memory.  rows [n, >= col0 + heads * (2 dim + 2 vdim)] hold q | k | v | gate; gates
+    float32 [n, 2 heads] the input gates' rows and then the forget gates' (``gate_bias`` float32 [2 heads] is added); state
+    float32 [slots, heads, dim, vdim + 1] (the memory and, as its last column, the normalizer) and m_state float32 [slots,
+    heads] (the running maximum) are read and left updated.  Returns [n, heads * vdim]: every head's output over its
+    denominator, unit-normed per head, times ``norm_w`` and the sigmoid of the gate.  ``chunk``: see ``mlstm_chunk``."""
+    what = "mlstm"
+    _dev(what, rows, gates, gate_bias, norm_w, state, m_state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    _i32(what, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    n = rows.shape[0]
+    in_rows = heads * (2 * dim + 2 * vdim)
+    _need(rows.dim() == 2 and col0 >= 0 and rows.shape[1] >= col0 + in_rows and n == ctx.n_tokens, f"{what}: rows {tuple(rows.shape)} from column {col0} "
+          f"are not [{ctx.n_tokens}, {heads} * (2*{dim} + 2*{vdim})]")
+    _need(gates.shape == (n, 2 * heads) and gates.dtype == F32, f"{what}: the gates' rows are float32 [{n}, {2 * heads}], not {gates.dtype} {tuple(gates.shape)}")
+    _need(gate_bias is None or (gate_bias.shape == (2 * heads,) and gate_bias.dtype == F32), f"{what}: the gates' bias is float32 [{2 * heads}]")
+    _need(norm_w.shape == (heads * vdim,) and norm_w.dtype == F32, f"{what}: the norm's weight is float32 [{heads * vdim}]")
+    _need(state.dim() == 4 and state.shape[1:] == (heads, dim, vdim + 1) and state.dtype == F32 and m_state.dim() == 2
+          and m_state.shape == (state.shape[0], heads) and m_state.dtype == F32,
+          f"{what}: state {tuple(state.shape)} {state.dtype} / {tuple(m_state.shape)} is not float32 [slots, {heads}, {dim}, {vdim + 1}] / [slots, {heads}]")
+    lib = mlstm_lib()
+    out = torch.empty((n, heads * vdim), dtype=rows.dtype, device=rows.device)
+    chunk = mlstm_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
+    qk = torch.empty((n, heads, 2, lib.palm_mlstm_pad(dim)), dtype=F32, device=rows.device)
+    coef = torch.empty((n, heads, 4), dtype=F32, device=rows.device)
+    starts = keeps = None
+    if chunk:
+        max_chunks = -(-ctx.max_new // chunk)
+        starts = torch.empty((ctx.n_seqs * max_chunks, heads, dim, vdim + 1), dtype=F32, device=rows.device)
+        keeps = torch.empty((ctx.n_seqs * max_chunks, heads), dtype=F32, device=rows.device)
+    library.call(lib, "palm_mlstm", _stream(), _p(rows), _code(rows, what), rows.shape[1], col0, col0 + heads * dim, col0 + 2 * heads * dim,
+                 col0 + 2 * heads * dim + heads * vdim, _p(gates), _p(gate_bias), float(cap), float(q_scale), _p(norm_w), float(eps), _p(state),
+                 _p(m_state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out), int(ctx.max_new),
+                 chunk, _p(starts), _p(keeps), n, _p(qk), _p(coef))
     return out

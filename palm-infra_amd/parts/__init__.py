@@ -1,8 +1,9 @@
 """The parts that layers are put together from: norms, position encodings, mixers, feed-forwards,
 blocks, and the embedding and head at the two ends."""
-from .base import (CATEGORIES, Builder, StepContext, cache_needs, context_ints, make_context, part_class, register_part)
+from .base import (CATEGORIES, Builder, StepContext, cache_needs, cache_needs_beside_shared, context_ints, make_context, part_class,
+                   register_part)
 from . import (norm, position, attention, feedforward, block, embedding, retention, selective_scan,  # noqa: F401  (registers the kinds)
-               differential_attention, delta_rule, latent_attention, sink_attention, parallel)
+               differential_attention, delta_rule, latent_attention, sink_attention, parallel, mlstm)
 from .linear import Linear
 from .residual import Prenormed, ResidualSink, WeightedSum, as_tensor, run_branch
 

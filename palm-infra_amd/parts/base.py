@@ -64,6 +64,15 @@ def cache_needs(spec: PartSpec) -> list:
     return list(fn(spec)) if fn else []
 
 
+def cache_needs_beside_shared(spec: PartSpec) -> list:
+    """What the part keeps of its own when its run-order entry reads another entry's storage (``cache_of``): nothing, unless
+    the part's class says otherwise with a static ``cache_needs_beside_shared(spec)`` (a mixer that borrows keys and values
+    but has a state of its own projections)."""
+    cls = part_class(spec.category, spec.kind)
+    fn = getattr(cls, "cache_needs_beside_shared", None)
+    return list(fn(spec)) if fn else []
+
+
 class Builder:
     """Builds parts from descriptions; hands them their parameters and the run's precision."""
 

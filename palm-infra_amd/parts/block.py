@@ -21,12 +21,16 @@ scaled add and the norm that reads the stream next are one kernel.
 ("layer scale").  A layer may have no feed-forward.  A branch may hand back a sum that is still to be made (the sides of
 parallel mixers with their weights); the terms, the vector, the 32-bit add and the norm that reads the stream next are
 one kernel.
+
+``hyper_connections``: the residual stream runs in S copies x_1 .. x_S.  A sublayer reads u = sum_s in[s] x_s through its norm
+(a ``streams_in`` reader), and its output y goes into all streams at once, x_t <- sum_s mix[s, t] x_s + out[t] y (every new
+stream from the old ones).  A layer may have no feed-forward.  The write of one sublayer and the read of the next are one kernel.
 """
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import cache_needs, register_part
-from .norm import PassThrough
+from .base import cache_needs, cache_needs_beside_shared, register_part
+from .norm import PassThrough, StreamsReader
 from .residual import ResidualSink, WeightedSum, as_tensor, run_branch
 
 
@@ -196,3 +200,54 @@ class ScaledPreNormBlock:
         h = self._add(x, y, self.mixer_scale, self.feed_forward_norm, None)
         y = self.feed_forward.forward(h, ctx)
         return self._add(x, y, self.feed_forward_scale, sink.norm, sink.rows)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionsBlock:
+    def __init__(self, spec, builder):
+        self.streams = int(spec.params["streams"])
+        self.mixer_norm = builder.build(spec.parts["mixer_norm"])
+        self.mixer = builder.build(spec.parts["mixer"])
+        self.mixer_mix, self.mixer_out = builder.tensor(spec, "mixer_mix"), builder.tensor(spec, "mixer_out")
+        self.feed_forward = builder.build(spec.parts["feed_forward"]) if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"]) if self.feed_forward is not None else None
+        self.feed_forward_mix = builder.tensor(spec, "feed_forward_mix") if self.feed_forward is not None else None
+        self.feed_forward_out = builder.tensor(spec, "feed_forward_out") if self.feed_forward is not None else None
+        S = self.streams
+        for mix, out_w in ((self.mixer_mix, self.mixer_out), (self.feed_forward_mix, self.feed_forward_out)):
+            if mix is not None and (mix.shape != (S, S) or out_w.shape != (S,)):
+                raise ValueError(f"{S} streams are written with weights [{S}, {S}] and [{S}], not {tuple(mix.shape)} and {tuple(out_w.shape)}")
+
+    @property
+    def capturable(self) -> bool:
+        parts = [self.mixer_norm, self.mixer] + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
+        return all(getattr(p, "capturable", False) for p in parts)
+
+    @staticmethod
+    def cache_needs(spec):
+        return cache_needs(spec.parts["mixer"])
+
+    @staticmethod
+    def cache_needs_beside_shared(spec):
+        return cache_needs_beside_shared(spec.parts["mixer"])
+
+    @property
+    def entry_norm(self):
+        return self.mixer_norm
+
+    @staticmethod
+    def _write(x, y, mix, out_w, reader, rows):
+        """The sublayer output y into the streams x; returns what ``reader`` makes of them, over ``rows``."""
+        if isinstance(reader, StreamsReader):
+            return reader.read(x, y, mix, out_w, rows=rows)
+        xs = x.view(x.shape[0], 1, x.shape[1]) if x.dim() == 2 else x
+        ops.streams_mix_norm(xs, y, mix, out_w, None, None, read=False)
+        return reader(x, rows=rows)
+
+    def forward(self, x, h, ctx, sink):
+        y = as_tensor(self.mixer.forward(as_tensor(h), ctx))
+        if self.feed_forward is None:
+            return self._write(x, y, self.mixer_mix, self.mixer_out, sink.norm, sink.rows)
+        h = self._write(x, y, self.mixer_mix, self.mixer_out, self.feed_forward_norm, None)
+        y = as_tensor(self.feed_forward.forward(h, ctx))
+        return self._write(x, y, self.feed_forward_mix, self.feed_forward_out, sink.norm, sink.rows)

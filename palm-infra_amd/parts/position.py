@@ -10,6 +10,9 @@ dim(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(f
 rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns with inv_i / factor * ramp_i +
 inv_i (1 - ramp_i), and cos and sin are both multiplied by 0.1 ln(factor) + 1.
 
+``scaling`` {kind: "linear", factor}: every frequency is divided by ``factor`` (positions count ``factor`` times slower);
+cos and sin keep their size.
+
 A position part hands the mixer cos/sin rows for the step's tokens, as the reference feeds its graph
 (models/qwen3.py:226-227); they are made once per step and shared by all layers that use the same
 part settings.
@@ -44,7 +47,9 @@ class Rotary:
         inv = np.float32(1.0) / np.power(np.float32(self.theta), np.float32(2.0) * i / np.float32(self.rotary_dim))
         self.magnitude = 1.0
         scaling = spec.params.get("scaling")
-        if scaling:
+        if scaling and scaling.get("kind") == "linear":
+            inv = (inv.astype(np.float64) / float(scaling["factor"])).astype(np.float32)
+        elif scaling:
             factor, original = float(scaling["factor"]), float(scaling["original"])
 
             def dim_of(turns: float) -> float:
@@ -56,7 +61,7 @@ class Rotary:
             inv = (inv.astype(np.float64) / factor * ramp + inv.astype(np.float64) * (1.0 - ramp)).astype(np.float32)
             self.magnitude = 0.1 * math.log(factor) + 1.0
         self.inv_freq = torch.from_numpy(inv.astype(np.float32)).to(builder.device)
-        self._key = ("rotary", self.rotary_dim, self.theta, tuple(sorted(scaling.items())) if scaling else None)
+        self._key = ("rotary", self.rotary_dim, self.theta, tuple(sorted((k, str(v)) for k, v in scaling.items())) if scaling else None)
 
     def tables(self, ctx):
         if self._key not in ctx.memo:
