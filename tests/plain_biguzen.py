@@ -247,3 +247,19 @@ def forward(raw, tensors, ids, layer_results=None):
             layer_results.append(xs.sum(0))
     x = xs.sum(0)
     return norm("final.norm", x) @ w["embed"].T
+
+
+def read_model(path):
+    """(raw config, tensors by name) of a model folder."""
+    import json
+    from pathlib import Path
+    from safetensors.torch import load_file
+    path = Path(path)
+    return json.loads((path / "config.json").read_text()), load_file(str(path / "model.safetensors"))
+
+
+def greedy(cfg, tensors, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(cfg, tensors, ids)[-1].argmax()))
+    return ids[len(prompt):]
