@@ -337,7 +337,22 @@ def _mixer_rooflines(raw: dict, tokens: int, batch: int, context: int) -> dict:
     hbm, mfma, vec = PEAK_HBM_GBS * 1e9, PEAK_FLOPS["bf16"], PEAK_FLOPS["fp32"]
     pairs = tokens * (tokens + 1) / 2.0
     out = {}
-    if "layers" in raw:
+    if raw.get("architecture") == "Biguzen":
+        for layer in raw["layers"]:
+            m = layer["mixer"]
+            if layer["type"] == "attention" and "palm_sink_attention" not in out:
+                w = m["mask"]["size"] if m.get("mask") else tokens
+                seen = sum(min(p + 1, w) for p in range(tokens))
+                out["palm_sink_attention_mfma"] = (2.0 * m["heads"] * (m["dim"] + m["vdim"]) * seen, mfma, None, None)
+                out["palm_sink_attention"] = (None, None, 2.0 * batch * min(context, w) * m["kv_heads"] * (m["dim"] + m["vdim"]), hbm)
+            elif layer["type"] == "mlstm" and "palm_mlstm" not in out:
+                per = m["heads"] * m["dim"] * (m["vdim"] + 1)          # two multiply-adds for every element of the memory and token
+                out["palm_mlstm"] = (4.0 * tokens * per, vec, 2.0 * 4 * batch * per, hbm)
+            f = layer.get("mlp")
+            if f and f["kind"] == "moe" and "palm_moe_experts" not in out:                 # plain experts: two matrices each
+                out["palm_moe_experts"] = (None, None, 2.0 * batch * f["router"]["top"] * 2 * f["expert"]["ff"] * raw["width"], hbm)
+                out["palm_moe_grouped"] = (2.0 * tokens * f["router"]["top"] * 2 * f["expert"]["ff"] * raw["width"], mfma, None, None)
+    elif "layers" in raw:
         for layer in raw["layers"]:
             m = layer["mixer"]
             if layer["type"] == "retention" and "palm_retention" not in out:
@@ -461,7 +476,18 @@ def _matalix_bench(args, record) -> dict:
     return record["sizes"]["matalix-2048"]["matalix"]
 
 
-DESIGNS = {"matalix": ("Matalix presets beside Sebesun presets of equal width and depth", _matalix_bench),
+def _biguzen_bench(args, record) -> dict:
+    """The Biguzen presets beside the Matalix presets of the same width and depth (the closest design here: the same attention
+    kernels with a window, a sink and a gate, and a recurrence over a matrix per head)."""
+    for width in ("2048", "4096"):
+        record["sizes"][f"biguzen-{width}"] = {
+            "biguzen": design_points(preset_dict(f"biguzen-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT),
+            "matalix": design_points(preset_dict(f"matalix-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT)}
+    return record["sizes"]["biguzen-2048"]["biguzen"]
+
+
+DESIGNS = {"biguzen": ("Biguzen presets beside Matalix presets of equal width and depth", _biguzen_bench),
+           "matalix": ("Matalix presets beside Sebesun presets of equal width and depth", _matalix_bench),
            "sebesun": ("Sebesun presets beside Qwen3 models of equal width and depth", _sebesun_bench),
            "pazilorn": ("Pazilorn presets beside Sebesun presets of equal width and depth", _pazilorn_bench)}
 
@@ -498,7 +524,7 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="tokens of the timed prompt (2,048 is the workload's; others serve profiles of longer prompts)")
     ap.add_argument("--design", help="instead of the default workload: another design's presets beside its closest relative "
-                    "of equal width and depth ('sebesun' beside Qwen3, 'pazilorn' and 'matalix' beside Sebesun)")
+                    "of equal width and depth ('sebesun' beside Qwen3, 'pazilorn' and 'matalix' beside Sebesun, 'biguzen' beside Matalix)")
     args = ap.parse_args(argv)
     if args.design:
         if args.gpus != 1:

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
     const int* __restrict__ tok_slot, const int* __restrict__ positions, int norm_mode, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
     int heads, int kv_heads, int dim, int vdim, int write_cache, int pairing,
-    const float* __restrict__ conv_w, int taps, const float* __restrict__ conv_state, int conv_channels) {
+    const float* __restrict__ conv_w, int taps, float* __restrict__ conv_state, int conv_channels, int fuse_state) {
     __shared__ float scratch[16];
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
@@ -123,6 +123,18 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
         for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x)
             v_cache[((size_t)page * kv_heads * vdim + i) * PAGE_TOKENS + at] = from_float<T>(value(v_off + i, q_size + k_size + i, v_b ? v_b + i : nullptr));
     }
+    // Every sequence of the step brings one token: this block is the only one that touches its sequence's state, and moves
+    // it on by its token once all the block's reads of the old state are done.
+    if (fuse_state && taps > 1) {
+        __syncthreads();
+        float* stw = conv_state + (size_t)tok_slot[t] * (taps - 1) * conv_channels;
+        for (int c = threadIdx.x; c < conv_channels; c += blockDim.x) {
+            const int col = c < q_size ? q_off + c : c < q_size + k_size ? k_off + (c - q_size) : v_off + (c - q_size - k_size);
+            const float cur = to_float(row[col]) + (bias ? bias[c] : 0.f);
+            for (int j = 0; j + 2 < taps; ++j) stw[(size_t)j * conv_channels + c] = stw[(size_t)(j + 1) * conv_channels + c];
+            stw[(size_t)(taps - 2) * conv_channels + c] = cur;
+        }
+    }
 }
 
 // After the pass above has read the old state: the last taps - 1 inputs (projection plus bias) of each sequence, old ones
@@ -174,6 +186,8 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
     if (n_tokens == 0) return 0;
     // the convolution's channels: q, and k and v if this layer makes them
     const int conv_channels = heads * dim + (write_cache ? kv_heads * (dim + vdim) : 0);
+    // one token a sequence (a decode step): the pass moves the state on itself; else a second launch does, after all reads
+    const int fuse_state = taps > 1 && n_tokens == n_seqs;
     // a wave takes a head at a time: for few tokens (a decode step) as many waves as there are heads of q and k, within a
     // block's sixteen; many tokens fill the chip anyway
     const int threads = n_tokens >= 256 ? 256 : min(1024, max(256, WAVE * (heads + kv_heads)));
@@ -181,8 +195,8 @@ PALM_API int palm_sink_qkv_store(hipStream_t stream, const void* rows, int dtype
         sink_qkv_store_kernel<T><<<n_tokens, threads, 0, stream>>>((const T*)rows, stride, q_off, k_off, v_off, bias, (T*)q_out, (T*)k_cache,
                                                               (T*)v_cache, block_table, max_pages, tok_slot, positions, norm_mode, q_w, k_w,
                                                               eps, cos_t, sin_t, rot, heads, kv_heads, dim, vdim, write_cache, pairing,
-                                                              conv_w, taps, conv_state, conv_channels);
-        if (taps > 1)
+                                                              conv_w, taps, conv_state, conv_channels, fuse_state);
+        if (taps > 1 && !fuse_state)
             sink_conv_state_kernel<T><<<dim3((conv_channels + 255) / 256, n_seqs), 256, 0, stream>>>(
                 (const T*)rows, stride, q_off, k_off, v_off, heads * dim, kv_heads * dim, bias, conv_state, seq_slot, seq_new, cu_new,
                 conv_channels, taps));

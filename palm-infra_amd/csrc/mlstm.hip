@@ -10,15 +10,16 @@
 //   out_t = o_t / sqrt(mean_v(o_t^2) + eps) * w * sigmoid(gate_t)              (the unit norm is per head, w over all heads)
 //
 // S, n and m are 32-bit and kept per sequence; gates, their logarithms, exponentials, the sums over the state and the norm
-// are 32-bit whatever the rows' type.  n is kept as one more column of S (a value that is always one), so S and n are one
-// tensor [dim, vdim + 1] and the recurrence is one formula.
+// are 32-bit whatever the rows' type.  n is stored as one more column of S, so S and n are one tensor [dim, vdim + 1].
 //
 // Three passes.  `gates`: a wave per (sequence, head) walks over the new tokens 64 at a time; each lane makes its token's
 // i and f, the wave composes the maps m -> max(m + f, i) with a scan (they are closed under composition), and every token
 // gets its three factors: what S keeps, what it takes, and exp(-m).  `qk`: q (times its scale) and k as 32-bit rows padded
 // to the key size the main kernel is compiled for.  The main kernel: one block per (head, sequence), one thread per column
-// of [S | n], the thread keeps its column in registers and walks over the tokens; q and k of a token are the same for all
-// threads and reach them as scalars; outputs are finished a tile of tokens at a time.  A prompt and a single token run the
+// of S, the thread keeps its column in registers and walks over the tokens; q and k of a token are the same for all
+// threads: a wave reads them one value a lane and hands them to its lanes as scalars.  n lies across the lanes of every
+// wave the same way (the lane that holds k[d] holds n[d]), so n . q is one multiply-add a lane and a sum over the wave, and
+// no thread is spent on it; outputs are finished a tile of tokens at a time.  A prompt and a single token run the
 // same code, so a prompt leaves the state that its tokens one by one leave.
 //
 // Given the factors the recurrence is linear in S, so a long run of new tokens is cut into chunks that run side by side:
@@ -82,7 +83,7 @@ __global__ void mlstm_qk_kernel(const T* __restrict__ rows, int row_stride, int 
     o[pad] = to_float(rows[row * row_stride + k_off + h * dim + d]);
 }
 
-// Thread v < vdim owns column v of S, thread vdim the column n.  DMAX: the padded key size; MAXT: the most threads of a block.
+// Thread v owns column v of S.  DMAX: the padded key size; MAXT: the most threads of a block.
 template <typename T, int DMAX, int MAXT>
 __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, float* __restrict__ chunk_keep,
                                                      const T* __restrict__ rows, int row_stride, int v_off, int g_off, const float* __restrict__ qk,
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
                                                      const int* __restrict__ cu_new, int heads, int dim, int vdim, T* __restrict__ out) {
     __shared__ float red[ML_TILE][16];
     __shared__ float o_s[ML_TILE][MAXT];
-    __shared__ float floor_s[ML_TILE];
+    __shared__ float floor_s[ML_TILE], nq_s[ML_TILE];
     constexpr int QREGS = (DMAX + WAVE - 1) / WAVE;
     const int h = blockIdx.x, b = blockIdx.y / max_chunks, c = blockIdx.y % max_chunks;
     const int v = threadIdx.x;
@@ -101,14 +102,14 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
     const int n_new = mode == ML_WHOLE ? seq_tokens : min(chunk, seq_tokens - c * chunk);
     const int row0 = cu_new[b] + (mode == ML_WHOLE ? 0 : c * chunk);
     const int cols = vdim + 1;
-    const bool mine = v < cols, is_value = v < vdim;
+    const bool mine = v < vdim;
     float* sp = mode == ML_WHOLE ? state + (((size_t)seq_slot[b] * heads + h) * dim) * cols + v
                                  : starts + ((((size_t)b * max_chunks + c) * heads + h) * dim) * cols + v;
 
     // the reads are unconditional (of a row and a column that exist) and what does not belong is set to zero after
     float S[DMAX];
     {
-        const float* at = sp - v + min(v, cols - 1);
+        const float* at = sp - v + min(v, vdim - 1);
         const bool zero = mode == ML_LOCAL || !mine;
         if (dim == DMAX) {
             const size_t stride = (size_t)cols;
@@ -127,8 +128,17 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
         }
     }
 
-    // A token's inputs: the thread's value (one for the column n), its three factors, and of its q and k rows one value a
-    // lane, which the wave hands to all its lanes as scalars.  The next token's are read while this one's are used.
+    // n: the lane that holds k[d] of a token holds n[d]; every wave keeps a copy
+    float nreg[QREGS];
+#pragma unroll
+    for (int i = 0; i < QREGS; ++i) {
+        const int d = i * WAVE + lane;
+        const float n0 = (sp - v)[(size_t)min(d, dim - 1) * cols + vdim];
+        nreg[i] = (mode == ML_LOCAL || d >= dim) ? 0.f : n0;
+    }
+
+    // A token's inputs: the thread's value, its three factors, and of its q and k rows one value a lane, which the wave
+    // hands to all its lanes as scalars.  The next token's are read while this one's are used.
     const int vc = min(v, vdim - 1);
     auto read_token = [&](int t, float& vv, float4& f, float (&qv)[QREGS], float (&kv)[QREGS]) {
         const size_t row = (size_t)(row0 + t);
@@ -151,9 +161,15 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
             float vn, qn[QREGS], kn[QREGS];
             float4 fn;
             read_token(min(t0 + ti + 1, n_new - 1), vn, fn, qn, kn);
-            if (!is_value) vv = mine ? 1.f : 0.f;
+            if (!mine) vv = 0.f;
             const float keep = f.x, in = f.y * vv;
             kept *= keep;
+            float nq = 0.f;
+#pragma unroll
+            for (int i = 0; i < QREGS; ++i) {
+                nreg[i] = fmaf(keep, nreg[i], f.y * kv[i]);
+                if (i * WAVE + lane < DMAX) nq = fmaf(nreg[i], qv[i], nq);        // (a key size below a wave: the upper lanes repeat)
+            }
             float acc = 0.f;
 #pragma unroll
             for (int d = 0; d < DMAX; ++d) {
@@ -163,10 +179,11 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
                 acc = fmaf(S[d], qd, acc);
             }
             if (mode != ML_LOCAL) {
+                nq = wave_sum(nq);
                 o_s[ti][v] = acc;
-                const float ss = wave_sum(is_value ? acc * acc : 0.f);
+                const float ss = wave_sum(acc * acc);
                 if (lane == 0) red[ti][wave] = ss;
-                if (v == 0) floor_s[ti] = f.z;
+                if (v == 0) { floor_s[ti] = f.z; nq_s[ti] = nq; }
             }
             vv = vn;
             f = fn;
@@ -179,11 +196,11 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
             float total = 0.f;
             for (int w = 0; w < n_waves; ++w) total += red[ti][w];
             // o = acc / denom for every column of the head, so the head's sum of squares is the raw one over denom^2
-            const float denom = fmaxf(fabsf(o_s[ti][vdim]), floor_s[ti]) + 1e-6f;
+            const float denom = fmaxf(fabsf(nq_s[ti]), floor_s[ti]) + 1e-6f;
             const float inv = 1.0f / sqrtf(total / (denom * denom) / (float)vdim + eps);
             const size_t row = (size_t)(row0 + t0 + ti);
             const float gate = to_float(rows[row * row_stride + g_off + h * vdim + vc]);
-            if (is_value)
+            if (mine)
                 out[row * ((size_t)heads * vdim) + h * vdim + v] =
                     from_float<T>(o_s[ti][v] / denom * inv * norm_w[h * vdim + v] * (1.0f / (1.0f + expf(-gate))));
         }
@@ -197,6 +214,13 @@ __global__ __launch_bounds__(MAXT) void mlstm_kernel(int mode, int chunk, int ma
 #pragma unroll
             for (int d = 0; d < DMAX; ++d)
                 if (d < dim) sp[(size_t)d * cols] = S[d];
+        }
+    }
+    if (wave == 0 && n_new > 0 && mode != ML_FROM_STARTS) {
+#pragma unroll
+        for (int i = 0; i < QREGS; ++i) {
+            const int d = i * WAVE + lane;
+            if (d < dim) (sp - v)[(size_t)d * cols + vdim] = nreg[i];
         }
     }
     if (mode == ML_LOCAL && v == 0) chunk_keep[((size_t)b * max_chunks + c) * heads + h] = kept;
@@ -250,7 +274,7 @@ PALM_API int palm_mlstm(hipStream_t stream, const void* rows, int dtype, int row
                         int vdim, void* out, int max_new, int chunk, float* starts, float* chunk_keep, int n_tokens, float* qk, float* coef) {
     PALM_CHECK(n_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0, "mlstm: seqs=%d heads=%d dim=%d vdim=%d", n_seqs, heads, dim, vdim);
     PALM_CHECK(dim <= 256, "mlstm: a key size of %d exceeds 256", dim);
-    PALM_CHECK(vdim + 1 <= 1024, "mlstm: a value size of %d exceeds 1023", vdim);
+    PALM_CHECK(vdim <= 1024, "mlstm: a value size of %d exceeds 1024", vdim);
     PALM_CHECK(cap > 0.f, "mlstm: the gates' cap %f must be positive", cap);
     PALM_CHECK(chunk >= 0 && (chunk == 0 || (starts && chunk_keep && max_new > 0)), "mlstm: chunks of %d tokens need their starting states", chunk);
     PALM_CHECK(n_tokens == 0 || (qk && coef && gates && norm_w && state && m_state && out), "mlstm: rows, factors and state need their room");
@@ -258,7 +282,7 @@ PALM_API int palm_mlstm(hipStream_t stream, const void* rows, int dtype, int row
     const int max_chunks = chunk > 0 ? (max_new + chunk - 1) / chunk : 1;
     PALM_CHECK(heads <= 65535 && (long long)n_seqs * max_chunks <= 65535, "mlstm: %d heads / %d sequences x %d chunks are more than one launch takes",
                heads, n_seqs, max_chunks);
-    const int threads = (vdim + 1 + WAVE - 1) / WAVE * WAVE;
+    const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
     dim3 grid(heads, n_seqs * max_chunks);
     const int pad = palm_mlstm_pad(dim);
     const long long qk_threads = (long long)n_tokens * heads * pad;

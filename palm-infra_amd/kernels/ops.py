@@ -1782,6 +1782,8 @@ def streams_mix_norm(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor
             _need(norm_w is not None and norm_w.shape == (width,) and norm_w.dtype == F32 and (norm_b is None or (norm_b.shape == (width,) and norm_b.dtype == F32)),
                   f"{what}: the norm's vectors are float32 [{width}]")
         out = torch.empty((n_rows, width), dtype=out_dtype or F32, device=xs.device)
+    if rows is not None and n_rows == 0:
+        return out                                  # nothing is read, and a selection leaves the streams as they are
     library.call(streams_lib(), "palm_streams_mix_norm", _stream(), _p(xs), n, S, width, _p(y), _code(y, what) if y is not None else 0, _p(mix),
                  _p(out_w), _p(in_w), STREAM_NORMS[norm], _p(norm_w), _p(norm_b), float(alpha), float(eps), _p(rows), n_rows,
                  int(rows is None and y is not None), _p(out), _code(out, what + " out") if out is not None else 0)
