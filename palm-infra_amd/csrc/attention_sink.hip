@@ -62,7 +62,7 @@ __global__ __launch_bounds__(1024) void sink_qkv_store_kernel(
     // column `col` of the rows, which is channel `ch` of q | k | v, with its bias, through the convolution
     auto value = [&](int col, int ch, const float* b) {
         const float bias_c = b ? *b : 0.f;
-        if (taps <= 1) return to_float(row[col]) + bias_c;
+        if (taps <= 1) return (to_float(row[col]) + bias_c) * (taps == 1 ? conv_w[ch] : 1.f);      // (one tap: a factor a channel)
         float acc = 0.f;
         for (int j = 0; j < taps; ++j) {
             const int back = taps - 1 - j;

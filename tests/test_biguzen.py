@@ -330,7 +330,8 @@ def test_streams_are_written_and_read_in_one_pass(W, norm):
 
 @gpu
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps,pairing,own", [(3, "interleaved", True), (4, "interleaved", False), (2, "half_split", True), (0, "interleaved", True)])
+@pytest.mark.parametrize("taps,pairing,own", [(3, "interleaved", True), (4, "interleaved", False), (2, "half_split", True), (0, "interleaved", True),
+                                               (1, "interleaved", True)])
 def test_q_k_v_pass_bias_convolution_over_portions_rotation_and_pages(dtype, taps, pairing, own):
     """Two sequences of unequal lengths go through the pass in portions of unequal sizes (down to one token, and portions
     shorter than the convolution reaches back), into slots that another sequence used before; q and the pages' contents
