@@ -152,32 +152,44 @@ __global__ __launch_bounds__(MOE_THREADS) void expert_gate_up_kernel(const T* __
     const bool gated = form == 0;                   // else: up rows alone, through the exact gelu
     const TW* w = gate_up + (size_t)e * (gated ? 2 : 1) * ff * width;
     const int f_end = min(ff, (int)(blockIdx.x + 1) * rows_per_block);
-    for (int f = blockIdx.x * rows_per_block + wave; f < f_end; f += n_waves) {
-        const TW* gr = w + (size_t)f * width;
-        const TW* ur = gated ? w + (size_t)(ff + f) * width : gr;
+    // Two rows of the first matrix are under way at a time in both forms: an inner value's gate row and up row, or (plain)
+    // the up rows of two inner values, the wave's own and the one n_waves further on.
+    const int step = gated ? n_waves : 2 * n_waves;
+    for (int f = blockIdx.x * rows_per_block + wave; f < f_end; f += step) {
+        const int f2 = f + n_waves;                                     // (plain form) the second inner value; beyond the block's rows: not kept
+        const TW* ur = gated ? w + (size_t)(ff + f) * width : w + (size_t)f * width;
+        const TW* gr = gated ? w + (size_t)f * width : w + (size_t)min(f2, ff - 1) * width;
         float g = 0.f, u = 0.f;
         if (width % 8 == 0) {                       // rows start on 16 bytes: eight values a lane and read
             for (int d = lane * 8; d < width; d += WAVE * 8) {
                 float gv[8], uv[8];
                 load8(ur + d, uv);
-                if (gated) load8(gr + d, gv);
+                load8(gr + d, gv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const float hv = h_s[d + i];
-                    if (gated) g = fmaf(gv[i], hv, g);
+                    g = fmaf(gv[i], hv, g);
                     u = fmaf(uv[i], hv, u);
                 }
             }
         } else {
             for (int d = lane; d < width; d += WAVE) {
                 const float hv = h_s[d];
-                if (gated) g = fmaf(to_float(gr[d]), hv, g);
+                g = fmaf(to_float(gr[d]), hv, g);
                 u = fmaf(to_float(ur[d]), hv, u);
             }
         }
         u = wave_sum(u);
-        if (gated) g = wave_sum(g);
-        if (lane == 0) mid[((size_t)t * top + c) * ff + f] = gated ? g / (1.0f + expf(-g)) * u : moe_gelu_erf(u);
+        g = wave_sum(g);
+        if (lane == 0) {
+            float* m = mid + ((size_t)t * top + c) * ff;
+            if (gated) {
+                m[f] = g / (1.0f + expf(-g)) * u;
+            } else {
+                m[f] = moe_gelu_erf(u);
+                if (f2 < f_end) m[f2] = moe_gelu_erf(g);
+            }
+        }
     }
 }
 
