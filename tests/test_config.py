@@ -129,7 +129,8 @@ def test_run_order_is_data_and_is_checked():
 def test_named_sizes_are_data_and_load():
     from palm_infra_amd.config import ConfigError, config_source, preset_dict, preset_names
     assert {"tiny-a", "tiny-b", "qwen3-8b", "qwen3-14b", "qwen3-32b", "tiny-sebesun", "sebesun-2048", "sebesun-4096",
-            "tiny-pazilorn", "pazilorn-2048", "pazilorn-4096", "tiny-matalix", "matalix-2048", "matalix-4096"} <= set(preset_names())
+            "tiny-pazilorn", "pazilorn-2048", "pazilorn-4096", "tiny-matalix", "matalix-2048", "matalix-4096",
+            "tiny-biguzen", "biguzen-2048", "biguzen-4096"} <= set(preset_names())
     for name in preset_names():
         cfg = config_from_dict(preset_dict(name))
         raw = preset_dict(name)
